@@ -1,0 +1,47 @@
+"""One registry from an architecture's name (config.json "architectures"[0]) to
+its configuration class; the configuration's ``plan()`` is its model recipe.
+
+The reference imports its model class directly (model/inference_paged.py:47) and
+picks engines from a dict (model/server.py:79-85); here the model folder's own
+config.json decides, everywhere in the framework.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+from .qwen3 import ConfigError, Qwen3Config
+
+_ARCHITECTURES = {}
+
+
+def register_architecture(name: str, config_cls) -> None:
+    """``config_cls`` needs ``from_dict(dict)``, ``to_dict()`` and ``plan() -> ModelPlan``."""
+    _ARCHITECTURES[name] = config_cls
+
+
+def known_architectures():
+    return sorted(_ARCHITECTURES)
+
+
+def config_class_for(name: str):
+    try:
+        return _ARCHITECTURES[name]
+    except KeyError:
+        raise ConfigError(f"unknown architecture {name!r}; known: {known_architectures()}") from None
+
+
+def load_config(folder):
+    """Read ``folder/config.json`` and return the typed configuration it names."""
+    path = Path(folder) / "config.json"
+    if not path.is_file():
+        raise ConfigError(f"{path} not found")
+    raw = json.loads(path.read_text())
+    archs = raw.get("architectures")
+    if not archs:
+        raise ConfigError(f"{path} has no 'architectures' entry; known: {known_architectures()}")
+    return config_class_for(archs[0]).from_dict(raw)
+
+
+register_architecture("Qwen3ForCausalLM", Qwen3Config)

@@ -1,0 +1,77 @@
+"""Grouped-query attention over paged keys and values.
+
+Formulas (model/qwen/qwen_kv_paged.py:147-175): q, k, v projections without bias,
+heads packed by index; per-head RMSNorm of q and k, then the position encoding;
+k and v go to the cache at the token's position; a query at position p in head h
+scores the keys 0..p (or the last ``window`` of them) of kv head h // G with
+``scale * <q, k>``, softmax in float32, and the weighted values are concatenated
+by head and projected by o_proj. The reference attends within the prompt only
+(qwen_kv_paged.py:167-173); here every query reads the pages, so a prompt may be
+cut anywhere.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import AttentionSpec
+from .registry import PagedKV, TensorDecl, build_part, register_part
+
+
+class PagedAttention:
+    @staticmethod
+    def tensors(spec: AttentionSpec):
+        q, kv, D = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.head_dim
+        t = {"q_proj.weight": TensorDecl((q, spec.hidden)),
+             "k_proj.weight": TensorDecl((kv, spec.hidden)),
+             "v_proj.weight": TensorDecl((kv, spec.hidden)),
+             "o_proj.weight": TensorDecl((spec.hidden, q))}
+        if spec.qk_norm is not None:
+            t["q_norm.weight"] = TensorDecl((D,), "vector")
+            t["k_norm.weight"] = TensorDecl((D,), "vector")
+        return t
+
+    @staticmethod
+    def cache_need(spec: AttentionSpec):
+        return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window)
+
+    def __init__(self, spec: AttentionSpec, tensors, ops):
+        self.spec, self.ops = spec, ops
+        if spec.qk_norm is not None and spec.qk_norm.dim != spec.head_dim:
+            raise ValueError("qk_norm runs over head_dim")
+        # One operand for the three projections: rows [q heads | k heads | v heads].
+        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
+                                tensors["v_proj.weight"]], dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        self.q_gain = tensors.get("q_norm.weight")
+        self.k_gain = tensors.get("k_norm.weight")
+        self.eps = spec.qk_norm.eps if spec.qk_norm is not None else 0.0
+        self.position = (build_part(spec.position, {}, ops)
+                         if spec.position is not None else None)
+
+    def forward(self, x, ctx, slot, write=True):
+        s, ops = self.spec, self.ops
+        Hq, Hkv, D = s.n_heads, s.n_kv_heads, s.head_dim
+        if write:
+            qkv = ops.linear(x, self.w_qkv)
+        else:
+            # Reading another step's cache: only the queries are needed.
+            qkv = ops.linear(x, self.w_qkv[: Hq * D])
+            Hkv = 0
+        rot = self.position.rotary() if hasattr(self.position, "rotary") else None
+        if self.position is None or rot is not None:
+            inv_freq, rotary_dim = rot if rot is not None else (None, 0)
+            q = ops.qk_norm_rope_write(
+                qkv, Hq, Hkv, D, self.q_gain, self.k_gain, self.eps, inv_freq, rotary_dim,
+                ctx.positions, ctx.token_rows, slot if write else None)
+        else:
+            # A position encoding without a fused form: norm, encode, then store.
+            q, k, v = ops.qk_norm_split(qkv, Hq, Hkv, D, self.q_gain, self.k_gain, self.eps)
+            self.position.apply(q, k, ctx.positions)
+            if write:
+                ops.kv_write(k, v, ctx.positions, ctx.token_rows, slot)
+        o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
+        return ops.linear(o, self.w_o)
+
+
+register_part(AttentionSpec, PagedAttention)

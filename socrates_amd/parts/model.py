@@ -1,0 +1,69 @@
+"""A decoder put together from a plan: embedding, blocks in the plan's order,
+final norm, output head (model/qwen/qwen_kv_paged.py:207-224).
+
+The forward pass runs exactly the tokens of one step batch, reads earlier
+tokens from the cache, and computes the final norm and the head only at the
+wanted places.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import ModelPlan
+from .block import block_tensors, build_block
+from .registry import TensorDecl, build_part, impl_of, tensors_of
+
+
+def expected_tensors(plan: ModelPlan):
+    """{tensor name on disk: TensorDecl} for the whole model."""
+    out = {plan.embedding_name: TensorDecl((plan.vocab_size, plan.hidden))}
+    for spec in plan.layers:
+        out.update(block_tensors(spec))
+    for local, decl in tensors_of(plan.final_norm).items():
+        out[f"{plan.final_norm_prefix}.{local}"] = decl
+    if plan.head_name is not None:
+        out[plan.head_name] = TensorDecl((plan.vocab_size, plan.hidden))
+    return out
+
+
+def cache_needs(plan: ModelPlan):
+    """The cache requirement of every cache slot, in slot order."""
+    needs = [None] * plan.n_cache_slots
+    for step in plan.order:
+        mixer = plan.layers[step.layer].mixer
+        need = impl_of(mixer).cache_need(mixer)
+        if needs[step.cache] is not None and needs[step.cache] != need and step.write:
+            raise ValueError(f"cache slot {step.cache} is claimed with two different needs")
+        if step.write:
+            needs[step.cache] = need
+        elif needs[step.cache] != need:
+            raise ValueError(f"run step of layer {step.layer} reads cache slot {step.cache}, "
+                             f"whose contents {needs[step.cache]} are not what it needs ({need})")
+    return needs
+
+
+class DecoderModel:
+    def __init__(self, plan: ModelPlan, weights, ops):
+        self.plan, self.ops = plan, ops
+        self.embed = weights[plan.embedding_name]
+        self.blocks = [build_block(spec, weights, ops) for spec in plan.layers]
+        norm_tensors = {local: weights[f"{plan.final_norm_prefix}.{local}"]
+                        for local in tensors_of(plan.final_norm)}
+        self.final_norm = build_part(plan.final_norm, norm_tensors, ops)
+        self.head = self.embed if plan.head_name is None else weights[plan.head_name]
+
+    def forward(self, ctx, cache):
+        """ctx: a StepContext on the device; cache: the CacheManager. Returns float32
+        logits [len(ctx.want_index), vocab]."""
+        ops = self.ops
+        residual = ops.embedding(ctx.token_ids, self.embed)
+        pending = None
+        for step in self.plan.order:
+            pending = self.blocks[step.layer].forward(
+                residual, pending, ctx, cache.slot(step.cache), step.write)
+        if ctx.n_want == 0:
+            # The cache is complete after the last block; no logits are asked for.
+            return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=ops.device)
+        h = self.final_norm.add_norm(residual, pending, rows=ctx.want_index)
+        return ops.linear(h, self.head, out_dtype=torch.float32)

@@ -1,0 +1,116 @@
+"""Weights from safetensors, by tensor name.
+
+The reference reads every shard named in model.safetensors.index.json into one
+dict and loads it strictly (model/qwen/qwen_kv_cont.py:35-42,
+model/inference_paged.py:73-75): a missing or unexpected name raises. Here a
+local folder holds either ``model.safetensors`` or an index with shards, names
+are the ones on disk (no renaming), and everything that is wrong is reported in
+one error: missing names, unexpected names and wrong shapes.
+
+Kept dtypes: matrix operands in the compute dtype, except that a tensor stored in
+32-bit floats stays 32-bit; gains and other vectors in float32 (exact from
+bfloat16); integer tables as int32.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import torch
+from safetensors import safe_open
+
+
+class WeightError(ValueError):
+    """Lists every missing tensor, unexpected tensor and wrong shape at once."""
+
+    def __init__(self, folder, missing, unexpected, wrong_shape, wrong_dtype=()):
+        self.missing, self.unexpected = sorted(missing), sorted(unexpected)
+        self.wrong_shape, self.wrong_dtype = list(wrong_shape), list(wrong_dtype)
+        lines = [f"weights in {folder} do not fit the model:"]
+        if self.missing:
+            lines.append(f"  missing ({len(self.missing)}): " + ", ".join(self.missing))
+        if self.unexpected:
+            lines.append(f"  unexpected ({len(self.unexpected)}): " + ", ".join(self.unexpected))
+        for name, want, got in self.wrong_shape:
+            lines.append(f"  wrong shape: {name} expected {list(want)}, found {list(got)}")
+        for name, got in self.wrong_dtype:
+            lines.append(f"  wrong dtype: {name} is {got}")
+        super().__init__("\n".join(lines))
+
+
+def _files_of(folder: Path):
+    """{tensor name: file} for a folder with one file or an index and shards."""
+    single, index = folder / "model.safetensors", folder / "model.safetensors.index.json"
+    if single.is_file():
+        files = [single]
+    elif index.is_file():
+        shards = sorted(set(json.loads(index.read_text())["weight_map"].values()))
+        files = [folder / s for s in shards]
+        absent = [str(f) for f in files if not f.is_file()]
+        if absent:
+            raise FileNotFoundError(f"shards named by {index} are absent: {absent}")
+    else:
+        raise FileNotFoundError(f"{folder} holds neither model.safetensors nor model.safetensors.index.json")
+    where = {}
+    for f in files:
+        with safe_open(str(f), framework="pt") as sf:
+            for name in sf.keys():
+                where[name] = f
+    return where
+
+
+_FLOATS = {"F64": torch.float64, "F32": torch.float32, "F16": torch.float16, "BF16": torch.bfloat16}
+_INTS = {"I64", "I32", "I16", "I8", "U8"}
+
+
+def kept_dtype(kind: str, stored: str, compute_dtype):
+    """The dtype a stored tensor is kept in; None if the stored dtype cannot serve."""
+    if kind == "int":
+        return torch.int32 if stored in _INTS else None
+    if stored not in _FLOATS:
+        return None
+    if kind == "vector":
+        return torch.float32
+    if compute_dtype == torch.float32 or stored in ("F32", "F64"):
+        return torch.float32
+    return compute_dtype
+
+
+def load_weights(folder, expected, compute_dtype, device):
+    """Read the tensors named in ``expected`` ({name: TensorDecl}) from ``folder``.
+
+    Returns {name: tensor on device}. Raises WeightError naming everything that
+    does not fit. As under the reference's strict load, an ``lm_head.weight`` in
+    the folder of a tied model is unexpected.
+    """
+    folder = Path(folder)
+    where = _files_of(folder)
+    missing = [n for n in expected if n not in where]
+    unexpected = [n for n in where if n not in expected]
+    wrong_shape, wrong_dtype = [], []
+    by_file = {}
+    for name, decl in expected.items():
+        if name in where:
+            by_file.setdefault(where[name], []).append((name, decl))
+    # First pass: shapes and dtypes only, nothing is read.
+    for f, items in by_file.items():
+        with safe_open(str(f), framework="pt") as sf:
+            for name, decl in items:
+                sl = sf.get_slice(name)
+                shape = tuple(sl.get_shape())
+                if shape != tuple(decl.shape):
+                    wrong_shape.append((name, decl.shape, shape))
+                if kept_dtype(decl.kind, sl.get_dtype(), compute_dtype) is None:
+                    wrong_dtype.append((name, sl.get_dtype()))
+    if missing or unexpected or wrong_shape or wrong_dtype:
+        raise WeightError(folder, missing, unexpected, wrong_shape, wrong_dtype)
+    out = {}
+    for f, items in by_file.items():
+        with safe_open(str(f), framework="pt") as sf:
+            for name, decl in items:
+                stored = sf.get_slice(name).get_dtype()
+                t = sf.get_tensor(name)
+                out[name] = t.to(device=device, dtype=kept_dtype(decl.kind, stored, compute_dtype)
+                                 ).contiguous()
+    return out
