@@ -1,0 +1,316 @@
+// Memory-bound kernels between the matrix products: embedding gather, RMSNorm with
+// the residual sum fused in, per-head QK-norm + rotary encoding + cache-page write,
+// SwiGLU. Statistics, angles and sums are float32; a result is rounded once when it
+// is stored in bfloat16. The residual stream is float32.
+//
+// Formulas: model/qwen/qwen_kv_cont.py:45-77, 250-266 and
+// model/qwen/qwen_kv_paged.py:111-127, 147-156 of the reference.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// out[n, :] = table[ids[n], :] as float32 (start of the residual stream)
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int d, int V) {
+    const int n = blockIdx.x;
+    int id = ids[n];
+    id = id < 0 ? 0 : (id >= V ? V - 1 : id);          // the host checks ids; never read outside
+    const T* row = table + (size_t)id * d;
+    float* o = out + (size_t)n * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+SOC_EXPORT int soc_embedding(const int* ids, const void* table, float* out, int N, int d, int V,
+                             int table_dtype, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (table_dtype == 0)
+        hipLaunchKernelGGL(embedding_kernel<float>, dim3(N), dim3(256), 0, stream, ids,
+                           (const float*)table, out, d, V);
+    else
+        hipLaunchKernelGGL(embedding_kernel<bf16>, dim3(N), dim3(256), 0, stream, ids,
+                           (const bf16*)table, out, d, V);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// In place: r = residual[n] + delta[n]; residual[n] = r; out[n] = r / sqrt(mean(r^2) + eps) * w.
+// With `rows`: n = rows[i], nothing is written back, out has one row per index.
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                   const float* __restrict__ w, T* __restrict__ out,
+                                   const int* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int n = rows ? rows[i] : i;
+    float* r = residual + (size_t)n * d;
+    const T* dl = delta ? delta + (size_t)n * d : nullptr;
+    T* o = out + (size_t)i * d;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < d; j += blockDim.x) {
+        float v = r[j];
+        if (dl) v += to_float(dl[j]);
+        if (!rows && dl) r[j] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    for (int j = threadIdx.x; j < d; j += blockDim.x) {
+        float v = r[j];
+        if (rows && dl) v += to_float(dl[j]);
+        o[j] = from_float<T>(v * inv * w[j]);
+    }
+}
+
+SOC_EXPORT int soc_add_rmsnorm(float* residual, const void* delta, const float* w, void* out,
+                               const int* rows, int n_out, int d, float eps, int dtype,
+                               hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    const int threads = d >= 2048 ? 512 : 256;
+    if (dtype == 0)
+        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, stream, residual,
+                           (const float*)delta, w, (float*)out, rows, d, eps);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, dim3(n_out), dim3(threads), 0, stream, residual,
+                           (const bf16*)delta, w, (bf16*)out, rows, d, eps);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Plain RMSNorm over rows of `dim` elements, one wave per row.
+template <typename T>
+__global__ void rmsnorm_rows_kernel(const T* __restrict__ x, const float* __restrict__ w,
+                                    T* __restrict__ out, int R, int dim, float eps) {
+    const int row = blockIdx.x * (blockDim.x / SOC_WAVE) + threadIdx.x / SOC_WAVE;
+    const int lane = threadIdx.x % SOC_WAVE;
+    if (row >= R) return;
+    const T* xr = x + (size_t)row * dim;
+    T* o = out + (size_t)row * dim;
+    float ss = 0.f;
+    for (int j = lane; j < dim; j += SOC_WAVE) { float v = to_float(xr[j]); ss += v * v; }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+    for (int j = lane; j < dim; j += SOC_WAVE) o[j] = from_float<T>(to_float(xr[j]) * inv * w[j]);
+}
+
+SOC_EXPORT int soc_rmsnorm(const void* x, const float* w, void* out, int R, int dim, float eps,
+                           int dtype, hipStream_t stream) {
+    if (R <= 0) return 0;
+    const int grid = (R + 3) / 4;
+    if (dtype == 0)
+        hipLaunchKernelGGL(rmsnorm_rows_kernel<float>, dim3(grid), dim3(256), 0, stream,
+                           (const float*)x, w, (float*)out, R, dim, eps);
+    else
+        hipLaunchKernelGGL(rmsnorm_rows_kernel<bf16>, dim3(grid), dim3(256), 0, stream,
+                           (const bf16*)x, w, (bf16*)out, R, dim, eps);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[n, j] = silu(gate_up[n, j]) * gate_up[n, ff + j],  silu(z) = z / (1 + exp(-z))
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < total; i += stride) {
+        const size_t n = i / ff, j = i % ff;
+        const float g = to_float(gate_up[n * 2 * ff + j]);
+        const float u = to_float(gate_up[n * 2 * ff + ff + j]);
+        out[i] = from_float<T>(u * (g / (1.0f + expf(-g))));
+    }
+}
+
+SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int dtype, hipStream_t stream) {
+    const size_t total = (size_t)N * ff;
+    if (total == 0) return 0;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (dtype == 0)
+        hipLaunchKernelGGL(swiglu_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           (const float*)gate_up, (float*)out, total, ff);
+    else
+        hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           (const bf16*)gate_up, (bf16*)out, total, ff);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Per token and head of a packed [q heads | k heads | v heads] row: RMSNorm over the head
+// (q and k only, if gains are given), rotate-half rotation at the token's position (q and k
+// only, if inv_freq is given), then store: q to q_out; k and v into the cache pages of the
+// token's row at its position, or to k_out / v_out when no pools are given.
+// One wave per head; a workgroup of 4 waves walks the heads of one token.
+#define SOC_MAX_HEAD 256
+
+template <typename T>
+__global__ void qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+                                    T* __restrict__ k_out, T* __restrict__ v_out,
+                                    T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                    const int* __restrict__ block_table, int table_width,
+                                    const int* __restrict__ token_rows,
+                                    const int* __restrict__ positions,
+                                    const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+                                    const float* __restrict__ inv_freq, int Hq, int Hkv, int D,
+                                    int rotary_dim, int BS, float eps) {
+    __shared__ float stage[4][SOC_MAX_HEAD];
+    const int n = blockIdx.x;
+    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    const int heads = Hq + 2 * Hkv;
+    const T* row = qkv + (size_t)n * heads * D;
+    const int pos = positions[n];
+    size_t page_base = 0;
+    if (k_pool) {
+        const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
+        page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;     // + kv_head * BS * D
+    }
+    const int half = rotary_dim / 2;
+    // The trip count is the same for all four waves so that the barriers below are uniform.
+    for (int h0 = 0; h0 < heads; h0 += 4) {
+        const int h = h0 + wave;
+        const bool active = h < heads;
+        const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
+        const T* x = row + (size_t)(active ? h : 0) * D;
+        float v[SOC_MAX_HEAD / SOC_WAVE];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+            const int e = lane + i * SOC_WAVE;
+            v[i] = e < D ? to_float(x[e]) : 0.f;
+            ss += v[i] * v[i];
+        }
+        const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+        if (gain && active) {
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+                const int e = lane + i * SOC_WAVE;
+                if (e < D) v[i] = v[i] * inv * gain[e];
+            }
+        }
+        if (inv_freq) {
+            const bool rotate = active && (is_q || is_k);
+#pragma unroll
+            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+                const int e = lane + i * SOC_WAVE;
+                if (e < D) stage[wave][e] = v[i];
+            }
+            __syncthreads();
+            if (rotate) {
+#pragma unroll
+            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+                const int e = lane + i * SOC_WAVE;
+                if (e < rotary_dim) {
+                    const int j = e < half ? e : e - half;
+                    const float partner = stage[wave][e < half ? e + half : e - half];
+                    float s, c;
+                    sincosf((float)pos * inv_freq[j], &s, &c);
+                    v[i] = e < half ? v[i] * c - partner * s : v[i] * c + partner * s;
+                }
+            }
+            }
+            __syncthreads();
+        }
+        if (!active) continue;
+        T* dst;
+        if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
+        else {
+            const int kvh = is_k ? h - Hq : h - Hq - Hkv;
+            if (k_pool) dst = (is_k ? k_pool : v_pool) + page_base + (size_t)kvh * BS * D;
+            else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
+        }
+#pragma unroll
+        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+            const int e = lane + i * SOC_WAVE;
+            if (e < D) dst[e] = from_float<T>(v[i]);
+        }
+    }
+}
+
+SOC_EXPORT int soc_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void* v_out, void* k_pool,
+                                void* v_pool, const int* block_table, int table_width,
+                                const int* token_rows, const int* positions, const float* q_gain,
+                                const float* k_gain, const float* inv_freq, int N, int Hq, int Hkv,
+                                int D, int rotary_dim, int BS, float eps, int dtype,
+                                hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (D > SOC_MAX_HEAD || D < 1) return (int)hipErrorInvalidValue;
+    if (dtype == 0)
+        hipLaunchKernelGGL(qk_norm_rope_kernel<float>, dim3(N), dim3(256), 0, stream, (const float*)qkv,
+                           (float*)q_out, (float*)k_out, (float*)v_out, (float*)k_pool, (float*)v_pool,
+                           block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
+                           Hq, Hkv, D, rotary_dim, BS, eps);
+    else
+        hipLaunchKernelGGL(qk_norm_rope_kernel<bf16>, dim3(N), dim3(256), 0, stream, (const bf16*)qkv,
+                           (bf16*)q_out, (bf16*)k_out, (bf16*)v_out, (bf16*)k_pool, (bf16*)v_pool,
+                           block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
+                           Hq, Hkv, D, rotary_dim, BS, eps);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rotation alone, in place on x [N, H, D].
+template <typename T>
+__global__ void rope_kernel(T* __restrict__ x, const int* __restrict__ positions,
+                            const float* __restrict__ inv_freq, int H, int D, int rotary_dim) {
+    const int n = blockIdx.x;
+    const int half = rotary_dim / 2;
+    const int pos = positions[n];
+    T* row = x + (size_t)n * H * D;
+    for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
+        const int h = i / half, j = i % half;
+        T* p = row + (size_t)h * D;
+        const float a = to_float(p[j]), b = to_float(p[j + half]);
+        float s, c;
+        sincosf((float)pos * inv_freq[j], &s, &c);
+        p[j] = from_float<T>(a * c - b * s);
+        p[j + half] = from_float<T>(b * c + a * s);
+    }
+}
+
+SOC_EXPORT int soc_rope(void* x, const int* positions, const float* inv_freq, int N, int H, int D,
+                        int rotary_dim, int dtype, hipStream_t stream) {
+    if (N <= 0 || H <= 0) return 0;
+    if (dtype == 0)
+        hipLaunchKernelGGL(rope_kernel<float>, dim3(N), dim3(256), 0, stream, (float*)x, positions,
+                           inv_freq, H, D, rotary_dim);
+    else
+        hipLaunchKernelGGL(rope_kernel<bf16>, dim3(N), dim3(256), 0, stream, (bf16*)x, positions,
+                           inv_freq, H, D, rotary_dim);
+    return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Store k, v [N, Hkv, D] into the pages of each token's row at its position.
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, const T* __restrict__ v,
+                                T* __restrict__ k_pool, T* __restrict__ v_pool,
+                                const int* __restrict__ block_table, int table_width,
+                                const int* __restrict__ token_rows,
+                                const int* __restrict__ positions, int Hkv, int D, int BS) {
+    const int n = blockIdx.x;
+    const int pos = positions[n];
+    const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
+    const size_t base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;
+    for (int i = threadIdx.x; i < Hkv * D; i += blockDim.x) {
+        const int h = i / D, e = i % D;
+        const size_t dst = base + (size_t)h * BS * D + e;
+        k_pool[dst] = k[(size_t)n * Hkv * D + i];
+        v_pool[dst] = v[(size_t)n * Hkv * D + i];
+    }
+}
+
+SOC_EXPORT int soc_kv_write(const void* k, const void* v, void* k_pool, void* v_pool,
+                            const int* block_table, int table_width, const int* token_rows,
+                            const int* positions, int N, int Hkv, int D, int BS, int dtype,
+                            hipStream_t stream) {
+    if (N <= 0 || Hkv <= 0) return 0;
+    if (dtype == 0)
+        hipLaunchKernelGGL(kv_write_kernel<float>, dim3(N), dim3(256), 0, stream, (const float*)k,
+                           (const float*)v, (float*)k_pool, (float*)v_pool, block_table, table_width,
+                           token_rows, positions, Hkv, D, BS);
+    else
+        hipLaunchKernelGGL(kv_write_kernel<bf16>, dim3(N), dim3(256), 0, stream, (const bf16*)k,
+                           (const bf16*)v, (bf16*)k_pool, (bf16*)v_pool, block_table, table_width,
+                           token_rows, positions, Hkv, D, BS);
+    return soc_last_error();
+}

@@ -1,0 +1,106 @@
+// Next-token choice from float32 logits, one workgroup per row.
+//
+// temperature 0: argmax, the lowest index among equal maxima (the reference is greedy
+// only: model/inference_paged.py:166, 193; ties: bench/day_8/equivalence.py:105-107).
+// temperature T > 0: an inverse-CDF draw from softmax(logits / T). The uniform number
+// comes from a counter-based hash of the request's seed and the number of draws it has
+// made, so a request's tokens do not depend on its neighbours in the batch. Every sum is
+// float32 and taken in a fixed order.
+#include "common.h"
+
+constexpr int SAMPLE_THREADS = 1024;
+
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+__device__ __forceinline__ float uniform_of(uint64_t seed, uint64_t draw) {
+    const uint64_t h = splitmix64(splitmix64(seed) ^ (draw * 0xD1342543DE82EF95ull));
+    return (float)(h >> 40) * (1.0f / 16777216.0f);          // 24 bits: exact in float32
+}
+
+struct MaxIdx { float v; int i; };
+
+__device__ __forceinline__ MaxIdx better(MaxIdx a, MaxIdx b) {
+    // NaN never wins; equal values keep the lower index
+    if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+    return a;
+}
+
+__device__ MaxIdx block_argmax(const float* __restrict__ x, int V, MaxIdx* scratch) {
+    MaxIdx best = {-INFINITY, 0x7fffffff};
+    for (int i = threadIdx.x; i < V; i += blockDim.x) best = better(best, MaxIdx{x[i], i});
+#pragma unroll
+    for (int m = SOC_WAVE / 2; m > 0; m >>= 1) {
+        MaxIdx o = {__shfl_xor(best.v, m, SOC_WAVE), __shfl_xor(best.i, m, SOC_WAVE)};
+        best = better(best, o);
+    }
+    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    if (lane == 0) scratch[wave] = best;
+    __syncthreads();
+    MaxIdx r = scratch[0];
+    for (int w = 1; w < blockDim.x / SOC_WAVE; ++w) r = better(r, scratch[w]);
+    __syncthreads();
+    if (r.i == 0x7fffffff) r.i = 0;                          // a row of NaN or -inf
+    return r;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+              const long long* __restrict__ seed, const long long* __restrict__ draws,
+              int* __restrict__ out, int V) {
+    __shared__ MaxIdx scratch[SAMPLE_THREADS / SOC_WAVE];
+    __shared__ float chunk_sum[SAMPLE_THREADS];
+    __shared__ int chosen;
+    const int row = blockIdx.x;
+    const float* x = logits + (size_t)row * V;
+    const MaxIdx top = block_argmax(x, V, scratch);
+    const float T = temperature ? temperature[row] : 0.f;
+    if (!(T > 0.f)) {
+        if (threadIdx.x == 0) out[row] = top.i;
+        return;
+    }
+    // Each thread owns a run of consecutive entries so that the CDF is taken in index order.
+    const int per = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int begin = min(V, (int)threadIdx.x * per), end = min(V, begin + per);
+    const float inv_T = 1.0f / T;
+    float s = 0.f;
+    for (int i = begin; i < end; ++i) s += expf((x[i] - top.v) * inv_T);
+    chunk_sum[threadIdx.x] = s;
+    if (threadIdx.x == 0) chosen = -1;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int t = 0; t < SAMPLE_THREADS; ++t) total += chunk_sum[t];
+        const float target = uniform_of((uint64_t)seed[row], (uint64_t)draws[row]) * total;
+        float run = 0.f;
+        int t = 0;
+        for (; t < SAMPLE_THREADS - 1; ++t) {
+            if (run + chunk_sum[t] > target) break;
+            run += chunk_sum[t];
+        }
+        // walk the owning run; the first entry whose cumulative weight exceeds the target
+        const int b = min(V, t * per), e = min(V, b + per);
+        int pick = top.i;
+        for (int i = b; i < e; ++i) {
+            run += expf((x[i] - top.v) * inv_T);
+            if (run > target) { pick = i; break; }
+        }
+        chosen = pick;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) out[row] = chosen;
+}
+
+// logits [n, V] float32; temperature [n] float32 or null (all greedy); seed, draws [n] int64.
+SOC_EXPORT int soc_sample(const float* logits, const float* temperature, const long long* seed,
+                          const long long* draws, int* out, int n, int V, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (V < 1) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(sample_kernel, dim3(n), dim3(SAMPLE_THREADS), 0, stream, logits, temperature,
+                       seed, draws, out, V);
+    return soc_last_error();
+}

@@ -1,0 +1,329 @@
+"""The kernel set: thin, checked Python wrappers over the HIP entry points.
+
+``HipKernels(dtype, device)`` is what every part computes with. It is the only
+kernel set in the package: there is no CPU or library path behind it, and it
+raises at construction if the GPU or a library is missing (the reference's
+``require_cuda_kernel``, model/kernels/__init__.py:82-92, has the same purpose).
+Wrappers check devices, dtypes, contiguity and shapes on the host before a kernel
+is launched, so that a wrong operand is an exception and not a memory fault.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+from .build import KernelBuildError, build_all, compile_library, load_library
+
+__all__ = ["HipKernels", "KernelBuildError", "build_all", "compile_library", "load_library"]
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _check(err, what):
+    if err != 0:
+        raise KernelError(f"{what}: HIP error {err}")
+
+
+P, I, F = c_void_p, c_int, c_float
+_EW_SIGNATURES = {
+    "soc_embedding": [P, P, P, I, I, I, I, P],
+    "soc_add_rmsnorm": [P, P, P, P, P, I, I, F, I, P],
+    "soc_rmsnorm": [P, P, P, I, I, F, I, P],
+    "soc_swiglu": [P, P, I, I, I, P],
+    "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
+    "soc_rope": [P, P, P, I, I, I, I, I, P],
+    "soc_kv_write": [P] * 5 + [I, P, P, I, I, I, I, I, P],
+}
+_GEMM_SIGNATURES = {
+    "soc_gemm_generic": [P, P, P, I, I, I, I, I, I, P],
+    "soc_gemm_bf16_mfma": [P, P, P, I, I, I, I, P],
+    "soc_gemm_bf16_skinny": [P, P, P, I, I, I, I, I, P],
+}
+_SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P]}
+_ATTENTION_SIGNATURES = {
+    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
+    "soc_attention_head_dim": [],
+}
+
+
+def _declare(lib, signatures):
+    for name, argtypes in signatures.items():
+        fn = getattr(lib, name)
+        fn.argtypes, fn.restype = argtypes, c_int
+
+
+class HipKernels:
+    def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
+        if dtype not in _DTYPE_CODE:
+            raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the HIP kernels are the only compute path "
+                              "(there is no CPU fallback)")
+        self.dtype, self.device = dtype, torch.device(device)
+        self.code = _DTYPE_CODE[dtype]
+        self._ew = load_library("elementwise")
+        self._gemm = load_library("gemm")
+        self._sampling = load_library("sampling")
+        self._attn = {}
+        _declare(self._ew, _EW_SIGNATURES)
+        _declare(self._gemm, _GEMM_SIGNATURES)
+        _declare(self._sampling, _SAMPLING_SIGNATURES)
+        self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
+
+    # -- helpers -----------------------------------------------------------------------------
+    def _stream(self):
+        return c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _want(self, t, name, dtype=None, shape=None):
+        if t.device.type != "cuda":
+            raise KernelError(f"{name} is on {t.device}, the kernels need it on the GPU")
+        if not t.is_contiguous():
+            raise KernelError(f"{name} is not contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} has dtype {t.dtype}, expected {dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    def _attention_lib(self, head_dim: int):
+        lib = self._attn.get(head_dim)
+        if lib is None:
+            if head_dim % 16 or not 16 <= head_dim <= 256:
+                raise KernelError(f"head size {head_dim}: the attention kernels take multiples of "
+                                  "16 from 16 to 256")
+            lib = load_library("attention", head_dim)
+            _declare(lib, _ATTENTION_SIGNATURES)
+            if lib.soc_attention_head_dim() != head_dim:
+                raise KernelError("attention library was built for another head size")
+            self._attn[head_dim] = lib
+        return lib
+
+    def prepare(self, head_dims=()):
+        """Compile and load, ahead of the first step, what a model with these head sizes needs."""
+        for d in head_dims:
+            self._attention_lib(d)
+
+    # -- embedding, norms, activation -------------------------------------------------------------
+    def embedding(self, ids, table):
+        self._want(ids, "ids", torch.int32)
+        self._want(table, "embedding table")
+        N, (V, d) = ids.numel(), table.shape
+        out = torch.empty((N, d), dtype=torch.float32, device=self.device)
+        _check(self._ew.soc_embedding(_ptr(ids), _ptr(table), _ptr(out), c_int(N), c_int(d), c_int(V),
+                                      c_int(_DTYPE_CODE[table.dtype]), self._stream()), "embedding")
+        return out
+
+    def add_rmsnorm(self, residual, delta, weight, eps, rows=None):
+        N, d = residual.shape
+        self._want(residual, "residual", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (d,))
+        if delta is not None:
+            self._want(delta, "delta", self.dtype, (N, d))
+        if rows is not None:
+            self._want(rows, "rows", torch.int32)
+        n_out = N if rows is None else rows.numel()
+        out = torch.empty((n_out, d), dtype=self.dtype, device=self.device)
+        _check(self._ew.soc_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
+                                        c_int(n_out), c_int(d), c_float(eps), c_int(self.code),
+                                        self._stream()), "add_rmsnorm")
+        return out
+
+    def rmsnorm(self, x, weight, eps):
+        dim = x.shape[-1]
+        self._want(x, "x", self.dtype)
+        self._want(weight, "norm weight", torch.float32, (dim,))
+        out = torch.empty_like(x)
+        _check(self._ew.soc_rmsnorm(_ptr(x), _ptr(weight), _ptr(out), c_int(x.numel() // dim), c_int(dim),
+                                    c_float(eps), c_int(self.code), self._stream()), "rmsnorm")
+        return out
+
+    def swiglu(self, gate_up):
+        self._want(gate_up, "gate_up", self.dtype)
+        N, two_ff = gate_up.shape
+        if two_ff % 2:
+            raise KernelError("gate_up needs an even last dimension")
+        out = torch.empty((N, two_ff // 2), dtype=self.dtype, device=self.device)
+        _check(self._ew.soc_swiglu(_ptr(gate_up), _ptr(out), c_int(N), c_int(two_ff // 2),
+                                   c_int(self.code), self._stream()), "swiglu")
+        return out
+
+    # -- matrix products ------------------------------------------------------------------------
+    def linear(self, x, w, out_dtype=None, n_waves=0):
+        """x [M, K] times w [N, K] transposed. float32 operands (either) take the plain
+        float32 kernel; bfloat16 pairs take the MFMA kernels."""
+        self._want(x, "x")
+        self._want(w, "weight")
+        if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+            raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(w.shape)}")
+        (M, K), N = x.shape, w.shape[0]
+        out_dtype = out_dtype or self.dtype
+        if x.dtype not in _DTYPE_CODE or w.dtype not in _DTYPE_CODE or out_dtype not in _DTYPE_CODE:
+            raise KernelError(f"linear: dtypes {x.dtype}, {w.dtype}, {out_dtype} are not supported")
+        out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        if M == 0:
+            return out
+        args = (_ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K))
+        both_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+        if both_bf16 and K % 8 == 0 and K >= 8:
+            if M <= 64:
+                err = self._gemm.soc_gemm_bf16_skinny(*args, c_int(_DTYPE_CODE[out_dtype]), c_int(n_waves),
+                                                      self._stream())
+            else:
+                err = self._gemm.soc_gemm_bf16_mfma(*args, c_int(_DTYPE_CODE[out_dtype]), self._stream())
+        else:
+            err = self._gemm.soc_gemm_generic(*args, c_int(_DTYPE_CODE[x.dtype]), c_int(_DTYPE_CODE[w.dtype]),
+                                              c_int(_DTYPE_CODE[out_dtype]), self._stream())
+        _check(err, f"linear [{M}x{K}] x [{N}x{K}]^T")
+        return out
+
+    # -- attention pieces ----------------------------------------------------------------------
+    def _qk(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps, inv_freq, rotary_dim, positions, token_rows,
+            slot, split_out):
+        N = qkv.shape[0]
+        self._want(qkv, "qkv", self.dtype, (N, (Hq + 2 * Hkv) * D))
+        if (q_gain is None) != (k_gain is None):
+            raise KernelError("q and k gains come together")
+        if q_gain is not None:
+            self._want(q_gain, "q gain", torch.float32, (D,))
+            self._want(k_gain, "k gain", torch.float32, (D,))
+        if inv_freq is not None:
+            if rotary_dim % 2 or not 2 <= rotary_dim <= D:
+                raise KernelError(f"rotary_dim {rotary_dim} does not fit head size {D}")
+            self._want(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+            self._want(positions, "positions", torch.int32, (N,))
+        q = torch.empty((N, Hq, D), dtype=self.dtype, device=self.device)
+        k = v = None
+        kp = vp = table = None
+        width = bs = 0
+        if slot is not None and Hkv:
+            self._check_slot(slot, Hkv, D)
+            self._want(positions, "positions", torch.int32, (N,))
+            self._want(token_rows, "token_rows", torch.int32, (N,))
+            kp, vp, table, width, bs = slot.k, slot.v, slot.block_table, slot.block_table.shape[1], slot.block_size
+        elif split_out and Hkv:
+            k = torch.empty((N, Hkv, D), dtype=self.dtype, device=self.device)
+            v = torch.empty((N, Hkv, D), dtype=self.dtype, device=self.device)
+        elif Hkv:
+            raise KernelError("keys and values need either a cache slot or split outputs")
+        if inv_freq is None and positions is None:
+            positions = torch.zeros((N,), dtype=torch.int32, device=self.device)
+        _check(self._ew.soc_qk_norm_rope(
+            _ptr(qkv), _ptr(q), _ptr(k), _ptr(v), _ptr(kp), _ptr(vp), _ptr(table), c_int(width),
+            _ptr(token_rows), _ptr(positions), _ptr(q_gain), _ptr(k_gain), _ptr(inv_freq), c_int(N),
+            c_int(Hq), c_int(Hkv), c_int(D), c_int(rotary_dim), c_int(bs), c_float(eps),
+            c_int(self.code), self._stream()), "qk_norm_rope")
+        return q, k, v
+
+    def _check_slot(self, slot, Hkv, D):
+        self._want(slot.k, "k pool", self.dtype)
+        self._want(slot.v, "v pool", self.dtype, slot.k.shape)
+        self._want(slot.block_table, "block table", torch.int32)
+        if slot.k.dim() != 4 or tuple(slot.k.shape[1:]) != (Hkv, slot.block_size, D):
+            raise KernelError(f"cache pool {tuple(slot.k.shape)} does not fit {Hkv} kv heads, "
+                              f"block size {slot.block_size}, head size {D}")
+
+    def qk_norm_rope_write(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps, inv_freq, rotary_dim,
+                           positions, token_rows, slot):
+        """Norm and rotate q and k, store k and v into the pages of ``slot`` (None: queries
+        only, ``Hkv`` 0). Returns q [N, Hq, D]."""
+        return self._qk(qkv, Hq, Hkv, D, q_gain, k_gain, eps, inv_freq, rotary_dim, positions,
+                        token_rows, slot, False)[0]
+
+    def qk_norm_split(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps):
+        """Norm q and k only; returns q, k, v as separate tensors."""
+        return self._qk(qkv, Hq, Hkv, D, q_gain, k_gain, eps, None, 0, None, None, None, True)
+
+    def rope(self, x, positions, inv_freq, rotary_dim):
+        N, H, D = x.shape
+        self._want(x, "x", self.dtype)
+        self._want(positions, "positions", torch.int32, (N,))
+        if rotary_dim % 2 or not 2 <= rotary_dim <= D:
+            raise KernelError(f"rotary_dim {rotary_dim} does not fit head size {D}")
+        self._want(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+        _check(self._ew.soc_rope(_ptr(x), _ptr(positions), _ptr(inv_freq), c_int(N), c_int(H), c_int(D),
+                                 c_int(rotary_dim), c_int(self.code), self._stream()), "rope")
+
+    def kv_write(self, k, v, positions, token_rows, slot):
+        N, Hkv, D = k.shape
+        self._want(k, "k", self.dtype)
+        self._want(v, "v", self.dtype, k.shape)
+        self._want(positions, "positions", torch.int32, (N,))
+        self._want(token_rows, "token_rows", torch.int32, (N,))
+        self._check_slot(slot, Hkv, D)
+        _check(self._ew.soc_kv_write(_ptr(k), _ptr(v), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+                                     c_int(slot.block_table.shape[1]), _ptr(token_rows), _ptr(positions),
+                                     c_int(N), c_int(Hkv), c_int(D), c_int(slot.block_size),
+                                     c_int(self.code), self._stream()), "kv_write")
+
+    def plan_splits(self, n_tokens, n_kv_heads, group, max_keys):
+        """How the keys of one token are cut into splits so that the launch fills the GPU."""
+        if self.attention_splits is not None:
+            return self.attention_splits
+        chunk = 1 if group == 1 else 2 if group == 2 else 4 if group <= 4 else 8
+        base = n_tokens * n_kv_heads * ((group + chunk - 1) // chunk)
+        if base >= 1024 or max_keys <= 256:
+            return 1 << 30, 1
+        n = min((max_keys + 127) // 128, (1024 + base - 1) // base)
+        split_len = ((max_keys + n - 1) // n + 63) // 64 * 64
+        return split_len, (max_keys + split_len - 1) // split_len
+
+    def paged_attention(self, q, slot, ctx, scale, window=None):
+        """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""
+        N, Hq, D = q.shape
+        self._want(q, "q", self.dtype)
+        Hkv = slot.k.shape[1]
+        self._check_slot(slot, Hkv, D)
+        if Hq % Hkv:
+            raise KernelError(f"{Hq} query heads do not divide into {Hkv} kv heads")
+        self._want(ctx.positions, "positions", torch.int32, (N,))
+        self._want(ctx.token_rows, "token_rows", torch.int32, (N,))
+        lib = self._attention_lib(D)
+        out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
+        w = int(window) if window else 0
+        max_keys = ctx.max_ctx_len if not w else min(w, ctx.max_ctx_len)
+        split_len, n_splits = self.plan_splits(N, Hkv, Hq // Hkv, max_keys)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty((N, Hq, n_splits, D), dtype=torch.float32, device=self.device)
+            part_ml = torch.empty((N, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
+        step = 65535
+        for lo in range(0, N, step):
+            n = min(step, N - lo)
+            _check(lib.soc_paged_attention_tokens(
+                _ptr(q[lo:lo + n]), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+                c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows[lo:lo + n]),
+                _ptr(ctx.positions[lo:lo + n]), _ptr(out[lo:lo + n]),
+                _ptr(part_o[lo:lo + n]) if part_o is not None else None,
+                _ptr(part_ml[lo:lo + n]) if part_ml is not None else None,
+                c_int(n), c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w),
+                c_int(split_len), c_int(n_splits), c_int(self.code), self._stream()), "paged_attention")
+        return out
+
+    # -- sampling ------------------------------------------------------------------------------
+    def argmax(self, logits):
+        return self.sample(logits, None, None, None)
+
+    def sample(self, logits, temperature, seed, draws):
+        """logits [n, V] float32; temperature [n] float32 (0: greedy), seed and draws [n] int64.
+        Returns int32 [n]."""
+        n, V = logits.shape
+        self._want(logits, "logits", torch.float32)
+        if temperature is not None:
+            self._want(temperature, "temperature", torch.float32, (n,))
+            self._want(seed, "seed", torch.int64, (n,))
+            self._want(draws, "draws", torch.int64, (n,))
+        out = torch.empty((n,), dtype=torch.int32, device=self.device)
+        _check(self._sampling.soc_sample(_ptr(logits), _ptr(temperature), _ptr(seed), _ptr(draws), _ptr(out),
+                                         c_int(n), c_int(V), self._stream()), "sample")
+        return out

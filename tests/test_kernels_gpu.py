@@ -1,0 +1,364 @@
+"""Each HIP kernel alone against its plain PyTorch reference, at sizes other than the
+engine's tiny models: head sizes in steps of 16, odd numbers of heads and groups, widths
+and vocabularies that are no power of two. float32 compares tightly; bfloat16 compares
+with the float32 reference computed from the same bfloat16 inputs."""
+
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from torch_kernels import TorchKernels, uniform_of
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: dict(atol=2e-5, rtol=2e-5), torch.bfloat16: dict(atol=2e-2, rtol=2e-2)}
+
+
+@pytest.fixture(scope="module")
+def kernel_sets():
+    from socrates_amd.kernels import HipKernels
+    return {dt: (HipKernels(dt, DEV), TorchKernels(dt, DEV)) for dt in DTYPES}
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, dtype, **over):
+    tol = dict(TOL[dtype], **over)
+    torch.testing.assert_close(got.float(), want.float(), **tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,V,d", [(1, 7, 16), (5, 331, 72), (33, 1000, 2560)])
+def test_embedding(kernel_sets, dtype, N, V, d):
+    hip, ref = kernel_sets[dtype]
+    table = rnd((V, d), dtype, 1)
+    ids = torch.randint(0, V, (N,), dtype=torch.int32, device=DEV)
+    got = hip.embedding(ids, table)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got, ref.embedding(ids, table), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,d,eps", [(1, 64, 1e-6), (7, 72, 1e-5), (19, 2560, 1e-6), (3, 5000, 1e-2)])
+def test_add_rmsnorm(kernel_sets, dtype, N, d, eps):
+    hip, ref = kernel_sets[dtype]
+    w = (1 + 0.3 * torch.randn(d)).to(DEV)
+    res = rnd((N, d), torch.float32, 2, 0.05)          # small rows: eps matters
+    delta = rnd((N, d), dtype, 3, 0.05)
+    r1, r2 = res.clone(), res.clone()
+    close(hip.add_rmsnorm(r1, delta, w, eps), ref.add_rmsnorm(r2, delta, w, eps), dtype)
+    torch.testing.assert_close(r1, r2, atol=1e-7, rtol=1e-6)          # the residual was updated
+    r1, r2 = res.clone(), res.clone()
+    close(hip.add_rmsnorm(r1, None, w, eps), ref.add_rmsnorm(r2, None, w, eps), dtype)
+    torch.testing.assert_close(r1, res, atol=0, rtol=0)
+    rows = torch.tensor([N - 1, 0, N // 2], dtype=torch.int32, device=DEV)
+    r1 = res.clone()
+    close(hip.add_rmsnorm(r1, delta, w, eps, rows), ref.add_rmsnorm(res.clone(), delta, w, eps, rows), dtype)
+    torch.testing.assert_close(r1, res, atol=0, rtol=0)                # gather mode writes nothing back
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_rows_matches_library_routine(kernel_sets, dtype):
+    hip, _ = kernel_sets[dtype]
+    x = rnd((11, 5, 48), dtype, 4)
+    w = (1 + 0.2 * torch.randn(48)).to(DEV)
+    want = torch.nn.functional.rms_norm(x.float(), (48,), w, 1e-5)
+    close(hip.rmsnorm(x, w, 1e-5), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,ff", [(1, 128), (9, 200), (130, 9728)])
+def test_swiglu(kernel_sets, dtype, N, ff):
+    hip, _ = kernel_sets[dtype]
+    gu = rnd((N, 2 * ff), dtype, 5, 2.0)
+    want = torch.nn.functional.silu(gu[:, :ff].float()) * gu[:, ff:].float()
+    close(hip.swiglu(gu), want, dtype)
+    zero_gate = gu.clone()
+    zero_gate[:, :ff] = 0
+    assert hip.swiglu(zero_gate).abs().max() == 0       # silu is on the gate half
+
+
+@pytest.mark.parametrize("a_dt,w_dt,c_dt", [
+    (torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.float32, torch.bfloat16),
+    (torch.bfloat16, torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (3, 331, 72), (8, 2560, 4096), (17, 100, 200), (33, 257, 96),
+                                   (64, 1000, 2560), (65, 130, 264), (130, 384, 96), (300, 700, 1032),
+                                   (5, 77, 33)])
+def test_linear(kernel_sets, a_dt, w_dt, c_dt, M, N, K):
+    hip, _ = kernel_sets[a_dt]
+    x, w = rnd((M, K), a_dt, 6), rnd((N, K), w_dt, 7, K ** -0.5)
+    got = hip.linear(x, w, out_dtype=c_dt)
+    want = x.double() @ w.double().T
+    assert got.dtype == c_dt
+    if c_dt == torch.float32:
+        torch.testing.assert_close(got.double(), want, atol=3e-5, rtol=3e-5)
+    else:
+        torch.testing.assert_close(got.double(), want, atol=2e-2, rtol=2e-2)
+
+
+def test_linear_float32_is_not_reduced_precision(kernel_sets):
+    """Values that bfloat16 or a 19-bit matrix mode would round away survive."""
+    hip, _ = kernel_sets[torch.float32]
+    x = torch.full((4, 64), 1.0 + 2.0 ** -20, device=DEV)
+    w = torch.full((8, 64), 1.0 + 2.0 ** -20, device=DEV)
+    got = hip.linear(x, w)
+    want = 64 * (1.0 + 2.0 ** -20) ** 2
+    assert abs(got[0, 0].item() - want) < 1e-4 and abs(got[0, 0].item() - 64.0) > 5e-5
+
+
+def make_paged_case(lens, Hq, Hkv, D, bs, dtype, seed, width=None, spare=5):
+    """Random K/V scattered over shuffled pages, one cache row per sequence, with the
+    contiguous K/V of each row for the reference."""
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    need = sum(-(-n // bs) for n in lens)
+    pages = list(range(1, need + spare + 1))
+    rng.shuffle(pages)
+    width = width or max(-(-n // bs) for n in lens) + 1
+    k_pool = torch.randn(need + spare + 1, Hkv, bs, D, generator=g)
+    v_pool = torch.randn(need + spare + 1, Hkv, bs, D, generator=g)
+    table = torch.zeros(len(lens), width, dtype=torch.int32)
+    dense = []
+    for r, n in enumerate(lens):
+        nb = -(-n // bs)
+        mine = [pages.pop() for _ in range(nb)]
+        table[r, :nb] = torch.tensor(mine, dtype=torch.int32)
+        k = k_pool[mine].permute(1, 0, 2, 3).reshape(Hkv, nb * bs, D)[:, :n]
+        v = v_pool[mine].permute(1, 0, 2, 3).reshape(Hkv, nb * bs, D)[:, :n]
+        dense.append((k.to(dtype).float(), v.to(dtype).float()))
+    slot = SimpleNamespace(k=k_pool.to(dtype).to(DEV), v=v_pool.to(dtype).to(DEV),
+                           block_table=table.to(DEV), block_size=bs, window=None)
+    return slot, dense
+
+
+def ctx_for(token_rows, positions):
+    return SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+                           token_rows=torch.tensor(token_rows, dtype=torch.int32, device=DEV),
+                           max_ctx_len=max(positions) + 1)
+
+
+def dense_attention(q, dense, token_rows, positions, scale, window=None):
+    """Per token: plain softmax attention over the row's contiguous keys lo..p."""
+    N, Hq, D = q.shape
+    out = torch.empty(N, Hq * D)
+    for t in range(N):
+        k, v = dense[token_rows[t]]
+        p = positions[t]
+        lo = 0 if window is None else max(0, p - window + 1)
+        k, v = k[:, lo:p + 1], v[:, lo:p + 1]
+        G = Hq // k.shape[0]
+        o = torch.nn.functional.scaled_dot_product_attention(
+            q[t].float().cpu().view(k.shape[0], G, 1, D), k[:, None], v[:, None], scale=scale)
+        out[t] = o.reshape(Hq * D)
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,bs", [(4, 2, 16, 16), (8, 2, 32, 8), (6, 2, 48, 16), (5, 5, 80, 4),
+                                         (32, 8, 128, 16), (16, 1, 64, 32), (2, 1, 256, 16)])
+def test_paged_attention_decode_tokens(kernel_sets, dtype, Hq, Hkv, D, bs):
+    hip, _ = kernel_sets[dtype]
+    lens = [1, 15, 16, 17, 300, 1025]
+    slot, dense = make_paged_case(lens, Hq, Hkv, D, bs, dtype, seed=D)
+    rows, pos = list(range(len(lens))), [n - 1 for n in lens]
+    q = rnd((len(lens), Hq, D), dtype, 8)
+    want = dense_attention(q, dense, rows, pos, 0.3)
+    for splits in (None, (128, 9), (64, 17), (1 << 30, 1)):
+        hip.attention_splits = splits
+        got = hip.paged_attention(q, slot, ctx_for(rows, pos), 0.3)
+        close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+    hip.attention_splits = None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
+    """Tokens of one row at consecutive positions (a portion that starts mid-sequence)
+    beside single tokens of other rows, with and without a window."""
+    hip, _ = kernel_sets[dtype]
+    Hq, Hkv, D, bs = 6, 2, 32, 8
+    lens = [70, 9, 130]
+    slot, dense = make_paged_case(lens, Hq, Hkv, D, bs, dtype, seed=11)
+    rows = [0] * 30 + [1] + [2] * 5
+    pos = list(range(40, 70)) + [8] + list(range(125, 130))
+    q = rnd((len(rows), Hq, D), dtype, 9)
+    for window in (None, 1, 7, 16, 64):
+        want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
+        got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
+        close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,slot_idx", [(1, 0), (16, 15), (17, 16), (256, 255), (257, 256), (1024, 1023),
+                                        (1, 1), (15, 15), (16, 16), (255, 255), (256, 256), (1024, 1024),
+                                        (600, 127), (600, 128), (600, 255), (600, 256), (1100, 511),
+                                        (1100, 512), (2048, 0), (2048, 1536)])
+def test_attention_needles(kernel_sets, dtype, n, slot_idx):
+    """The reference's needle vectors (tests/test_kernel_cuda.py:70-107): q = 0 makes every
+    weight exactly 1/n; V is zero except one slot that holds 8 * (kv head + 1). The output is
+    8 * (head // G + 1) / n if that slot is read and exactly 0 if it lies past the end."""
+    hip, _ = kernel_sets[dtype]
+    Hq, Hkv, D, bs = 32, 8, 128, 16
+    nb = -(-max(n, slot_idx + 1) // bs)
+    pages = torch.randperm(nb + 5)[:nb] + 1
+    kp = torch.randn(nb + 6, Hkv, bs, D)
+    vp = torch.zeros(nb + 6, Hkv, bs, D)
+    for h in range(Hkv):
+        vp[pages[slot_idx // bs], h, slot_idx % bs] = 8.0 * (h + 1)
+    table = torch.zeros(1, 130, dtype=torch.int32)
+    table[0, :nb] = pages.to(torch.int32)
+    slot = SimpleNamespace(k=kp.to(dtype).to(DEV), v=vp.to(dtype).to(DEV), block_table=table.to(DEV),
+                           block_size=bs, window=None)
+    q = torch.zeros(1, Hq, D, dtype=dtype, device=DEV)
+    G = Hq // Hkv
+    head_val = torch.tensor([8.0 * (i // G + 1) for i in range(Hq)])
+    want = (head_val / n if slot_idx < n else torch.zeros(Hq))[:, None].expand(Hq, D).reshape(1, Hq * D)
+    for splits in (None, (128, 17), (256, 9), (512, 5)):
+        hip.attention_splits = splits
+        got = hip.paged_attention(q, slot, ctx_for([0], [n - 1]), 0.1)
+        torch.testing.assert_close(got.float().cpu(), want, atol=1e-4, rtol=8e-3)
+    hip.attention_splits = None
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_ignores_poison_past_the_end(kernel_sets, dtype):
+    """inf / NaN in slots past each row's length, and in the null page, change nothing
+    (tests/test_kernel_cuda.py:120-133)."""
+    hip, _ = kernel_sets[dtype]
+    lens = [20, 7, 300, 1025]
+    slot, _ = make_paged_case(lens, 8, 2, 64, 16, dtype, seed=5)
+    rows, pos = list(range(4)), [n - 1 for n in lens]
+    q = rnd((4, 8, 64), dtype, 10)
+    before = hip.paged_attention(q, slot, ctx_for(rows, pos), 0.125)
+    for r, n in enumerate(lens):
+        last = int(slot.block_table[r, (n - 1) // 16])
+        if n % 16:
+            slot.k[last, :, n % 16:] = float("inf")
+            slot.v[last, :, n % 16:] = float("nan")
+    slot.k[0] = float("nan")
+    slot.v[0] = float("inf")
+    after = hip.paged_attention(q, slot, ctx_for(rows, pos), 0.125)
+    assert torch.isfinite(after).all()
+    torch.testing.assert_close(after, before, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,rot", [(4, 2, 16, 16), (8, 2, 32, 32), (6, 2, 48, 48), (3, 1, 128, 64),
+                                          (2, 2, 256, 256)])
+def test_qk_norm_rope_write(kernel_sets, dtype, Hq, Hkv, D, rot):
+    from socrates_amd.cache import CacheManager
+    from socrates_amd.parts import PagedKV
+    hip, ref = kernel_sets[dtype]
+    N, bs = 21, 8
+    caches = [CacheManager([PagedKV(Hkv, D)], 3, 64, bs, 20, dtype, DEV) for _ in range(2)]
+    rows, pos = [], []
+    for c in caches:
+        for n_tok in (9, 1, 11):
+            r = c.open_row()
+            if n_tok == 11:
+                c.reserve(r, 30)
+                c.advance(r, 19)                   # this row continues at position 19
+            c.reserve(r, c.length(r) + n_tok)
+        c.sync()
+    for r, n_tok, start in ((0, 9, 0), (1, 1, 0), (2, 11, 19)):
+        rows += [r] * n_tok
+        pos += list(range(start, start + n_tok))
+    positions = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    token_rows = torch.tensor(rows, dtype=torch.int32, device=DEV)
+    qkv = rnd((N, (Hq + 2 * Hkv) * D), dtype, 12)
+    qg, kg = (1 + 0.2 * torch.randn(D)).to(DEV), (1 + 0.2 * torch.randn(D)).to(DEV)
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot))).to(DEV)
+    args = (qkv, Hq, Hkv, D, qg, kg, 1e-5, inv_freq, rot, positions, token_rows)
+    got = hip.qk_norm_rope_write(*args, caches[0].slot(0))
+    want = ref.qk_norm_rope_write(*args, caches[1].slot(0))
+    close(got, want, dtype)
+    close(caches[0].slot(0).k, caches[1].slot(0).k, dtype)
+    close(caches[0].slot(0).v, caches[1].slot(0).v, dtype, atol=0, rtol=0)
+    # the unfused pieces give the same
+    q2, k2, v2 = hip.qk_norm_split(qkv, Hq, Hkv, D, qg, kg, 1e-5)
+    hip.rope(q2, positions, inv_freq, rot)
+    hip.rope(k2, positions, inv_freq, rot)
+    close(q2, want, dtype)
+    fresh = CacheManager([PagedKV(Hkv, D)], 3, 64, bs, 20, dtype, DEV)
+    for n_tok in (9, 1, 30):
+        fresh.reserve(fresh.open_row(), n_tok)
+    fresh.sync()
+    # same pages as caches[1]: both allocate 1, 2, 3, ... in the same order
+    hip.kv_write(k2, v2, positions, token_rows, fresh.slot(0))
+    close(fresh.slot(0).k, caches[1].slot(0).k, dtype)
+
+
+def test_rope_properties(kernel_sets):
+    """Position 0 is the identity; pair norms are kept; <rope(q, m), rope(k, n)> depends on
+    m - n only; equals complex multiplication by e^{i pos theta^(-2j/D)}."""
+    hip, _ = kernel_sets[torch.float32]
+    D, theta = 32, 1e4
+    inv_freq = (1.0 / (theta ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    x = rnd((6, 1, D), torch.float32, 13)
+    y = x.clone()
+    hip.rope(y, torch.zeros(6, dtype=torch.int32, device=DEV), inv_freq, D)
+    torch.testing.assert_close(y, x, atol=0, rtol=0)
+    pos = torch.tensor([3, 10, 100, 1000, 4095, 7], dtype=torch.int32, device=DEV)
+    y = x.clone()
+    hip.rope(y, pos, inv_freq, D)
+    z = torch.complex(x[..., :D // 2].double(), x[..., D // 2:].double()) * torch.polar(
+        torch.ones(6, 1, D // 2, dtype=torch.float64, device=DEV),
+        (pos.float()[:, None, None] * inv_freq).double())
+    torch.testing.assert_close(y[..., :D // 2].double(), z.real, atol=1e-5, rtol=1e-5)
+    torch.testing.assert_close(y[..., D // 2:].double(), z.imag, atol=1e-5, rtol=1e-5)
+    q, k = rnd((1, 1, D), torch.float32, 14), rnd((1, 1, D), torch.float32, 15)
+    dots = []
+    for m, n in ((5, 2), (105, 102), (2003, 2000)):
+        a, b = q.clone(), k.clone()
+        hip.rope(a, torch.tensor([m], dtype=torch.int32, device=DEV), inv_freq, D)
+        hip.rope(b, torch.tensor([n], dtype=torch.int32, device=DEV), inv_freq, D)
+        dots.append((a * b).sum().item())
+    # float32 angles resolve position * 2^-24 radians: the invariance holds to that
+    bound = 4 * 2003 * 2.0 ** -24 * (q.norm() * k.norm()).item()
+    assert max(dots) - min(dots) < bound
+    assert abs(dots[0] - dots[1]) < 4 * 105 * 2.0 ** -24 * (q.norm() * k.norm()).item()
+
+
+def test_sampling(kernel_sets):
+    hip, ref = kernel_sets[torch.float32]
+    V = 151936
+    logits = rnd((5, V), torch.float32, 16, 3.0)
+    logits[1, 777] = logits[1, 12345] = 50.0            # a tie: the lower index wins
+    logits[2] = -1e30
+    logits[2, V - 1] = 0.0
+    assert hip.argmax(logits).tolist() == ref.argmax(logits).tolist()
+    assert hip.argmax(logits)[1].item() == 777
+    n = 64
+    lg = rnd((n, 331), torch.float32, 17, 2.0)
+    temp = torch.full((n,), 0.8, device=DEV)
+    temp[::7] = 0.0
+    seed = torch.arange(n, dtype=torch.int64, device=DEV) * 7919 + 1
+    draws = torch.arange(n, dtype=torch.int64, device=DEV) % 5
+    got = hip.sample(lg, temp, seed, draws).tolist()
+    want = ref.sample(lg, temp, seed, draws).tolist()
+    # the chosen token's CDF interval holds the uniform number (up to float32 rounding)
+    agree = 0
+    for i in range(n):
+        if temp[i] == 0:
+            assert got[i] == int(lg[i].argmax())
+            continue
+        p = torch.softmax(lg[i].double() / 0.8, -1).cpu()
+        cdf = torch.cumsum(p, -1)
+        u = uniform_of(int(seed[i]), int(draws[i]))
+        lo = cdf[got[i] - 1].item() if got[i] else 0.0
+        assert lo - 1e-5 <= u <= cdf[got[i]].item() + 1e-5
+        agree += got[i] == want[i]
+    assert agree >= n - 10 - 2
+    # same (seed, draw) gives the same token whatever else is in the batch
+    again = hip.sample(lg[10:20].contiguous(), temp[10:20].contiguous(), seed[10:20].contiguous(),
+                       draws[10:20].contiguous()).tolist()
+    assert again == got[10:20]
+    # temperature to zero converges to argmax
+    cold = hip.sample(lg, torch.full((n,), 1e-4, device=DEV), seed, draws)
+    assert cold.tolist() == lg.argmax(-1).tolist()

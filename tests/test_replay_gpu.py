@@ -1,0 +1,103 @@
+"""The engine's step function on the GPU against the plain implementation, under every
+way of cutting the same requests into steps, in float32 and in bfloat16."""
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import (TINIES, make_runner, random_prompts, replay, trace_mixed, trace_portions,
+                     trace_tail_decode, trace_whole, write_tiny)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# float32: the reference's own bound for whole-model logits (tests/test_paged_model.py: 1e-4).
+# bfloat16: activations are rounded to 8 bits of mantissa between kernels; logits of size ~2
+# come out within a few hundredths of the float32 oracle that uses the same weights.
+TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
+LENGTHS = [5, 17, 33, 70, 64, 129]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("replay_models")
+    return {name: write_tiny(base / name, tiny, seed=3 + i) for i, (name, tiny) in enumerate(TINIES.items())}
+
+
+@pytest.fixture(scope="module")
+def oracle(folders):
+    out = {}
+    for name, folder in folders.items():
+        cfg, w = plain.read_folder(folder)
+        prompts = random_prompts(LENGTHS, cfg["vocab_size"], seed=len(name))
+        out[name] = (prompts, {f"r{i}": plain.forward(cfg, w, p) for i, p in enumerate(prompts)})
+    return out
+
+
+def runner_for(folder, tiny, dtype, num_blocks):
+    from socrates_amd.kernels import HipKernels
+    return make_runner(folder, HipKernels(dtype, DEV), max_rows=4, max_len=256,
+                       block_size=tiny["block_size"], num_blocks=num_blocks)
+
+
+def compare(got, want, dtype, label):
+    tol = TOL[dtype]
+    for rid in want:
+        assert got[rid].shape == want[rid].shape, (label, rid)
+        bad = ((got[rid] - want[rid]).abs() > tol["atol"] + tol["rtol"] * want[rid].abs()).any(dim=-1)
+        if bad.any():
+            first = int(bad.nonzero()[0])
+            err = (got[rid][first] - want[rid][first]).abs().max().item()
+            raise AssertionError(f"{label} request {rid}: {int(bad.sum())} of {len(bad)} positions are "
+                                 f"off; the first is position {first} (max error {err:.3g})")
+
+
+CUTS = {
+    "whole": lambda prompts: trace_whole(prompts),
+    "tail32": lambda prompts: trace_tail_decode(prompts, 32),
+    "portions": lambda prompts: trace_portions(prompts, seed=1),
+    "mixed": lambda prompts: trace_mixed(prompts, seed=2),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("cut", list(CUTS))
+@pytest.mark.parametrize("name", list(TINIES))
+def test_cut_matches_plain(folders, oracle, name, cut, dtype):
+    prompts, want = oracle[name]
+    bs = TINIES[name]["block_size"]
+    # so few pages that finished requests' pages are used again: the four longest
+    # requests together, rounded up to pages, and nothing more
+    longest = sorted((len(p) for p in prompts), reverse=True)[:4]
+    num_blocks = sum(-(-n // bs) for n in longest)
+    runner = runner_for(folders[name], TINIES[name], dtype, num_blocks)
+    got = replay(runner, CUTS[cut](prompts))
+    compare(got, want, dtype, f"{name}/{cut}")
+    assert runner.cache.n_free_pages == num_blocks and not runner.cache.open_rows
+
+
+@pytest.mark.parametrize("name", list(TINIES))
+def test_bf16_cuts_agree_with_each_other(folders, oracle, name):
+    """Cutting changes only the order of a few float32 sums, so bfloat16 logits of the
+    same position differ between cuts by a few bfloat16 roundings, far less than they
+    differ from the float32 oracle."""
+    prompts, _ = oracle[name]
+    results = {}
+    for cut in ("whole", "mixed"):
+        runner = runner_for(folders[name], TINIES[name], torch.bfloat16, 64)
+        results[cut] = replay(runner, CUTS[cut](prompts))
+    for rid in results["whole"]:
+        torch.testing.assert_close(results["mixed"][rid], results["whole"][rid], atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_first_tokens_and_long_decode(folders, dtype):
+    """The first tokens of a sequence one by one (positions 0, 1, 2 ...), then a long
+    decode across many page edges."""
+    cfg, w = plain.read_folder(folders["B"])
+    prompt = random_prompts([200], cfg["vocab_size"], seed=9)[0]
+    want = plain.forward(cfg, w, prompt)
+    runner = runner_for(folders["B"], TINIES["B"], dtype, 32)
+    steps = [([("r0", prompt[t:t + 1], [0])], []) for t in range(len(prompt))]
+    got = replay(runner, steps)["r0"]
+    torch.testing.assert_close(got, want, **TOL[dtype])

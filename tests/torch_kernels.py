@@ -148,6 +148,6 @@ class TorchKernels:
             u = uniform_of(int(seed[i]), int(draws[i]))
             p = torch.softmax(logits[i].double() / T, dim=-1)
             cdf = torch.cumsum(p, dim=-1)
-            tok = int(torch.searchsorted(cdf, torch.tensor(u * float(cdf[-1]), dtype=cdf.dtype), right=True))
+            tok = int(torch.searchsorted(cdf, torch.tensor(u * float(cdf[-1]), dtype=cdf.dtype, device=cdf.device), right=True))
             out.append(min(tok, logits.shape[1] - 1))
         return torch.tensor(out, dtype=torch.int32, device=logits.device)
