@@ -1,0 +1,166 @@
+"""Decode and prefill throughput of the engine at Qwen3-4B size on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A step is one decode step of the engine: plan, run the batch through the model from
+the cache, sample, read the tokens back. Random weights (seeded), prompts of uniform
+random token ids, every request prefilled through the engine to a context of
+``--context`` tokens before timing. Prints one JSON line.
+"""
+
+import argparse
+import json
+import random
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+# Published MI355X peaks used for the roofline fractions.
+HBM_GBPS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=2560,
+                num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                intermediate_size=9728, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True)
+FULL_LAYERS = QWEN3_4B["num_hidden_layers"]
+
+
+def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_):
+    import torch
+
+    from socrates_amd.cache import CacheManager, blocks_for
+    from socrates_amd.config import Qwen3Config
+    from socrates_amd.engine import Engine, ModelRunner
+    from socrates_amd.kernels import HipKernels
+    from socrates_amd.parts import DecoderModel, cache_needs, expected_tensors
+    from socrates_amd.weights import random_tensors
+
+    config = Qwen3Config.from_dict(cfg_dict)
+    plan = config.plan()
+    ops = HipKernels(dtype, "cuda:0")
+    weights = random_tensors(expected_tensors(plan), seed, dtype=dtype, device="cuda:0")
+    model = DecoderModel(plan, weights, ops)
+    del weights
+    cache = CacheManager(cache_needs(plan), max_rows=max_batch, max_len=max_len, block_size=16,
+                         num_blocks=max_batch * blocks_for(max_len, 16), dtype=dtype, device="cuda:0")
+    runner = ModelRunner(model, cache)
+    engine = Engine(runner, max_batch=max_batch, max_len=max_len, max_new_tokens=max_len,
+                    chunk=2048, compile=compile_)
+    return config, engine
+
+
+def decode_rate(engine, batch, context, steps, warmup, vocab, seed):
+    """Prefill ``batch`` prompts of ``context`` - 1 tokens through the engine, then time
+    ``steps`` decode steps. Returns (tokens per second, ms per step)."""
+    import torch
+    rng = random.Random(seed)
+    from socrates_amd.sampling import SamplingParams
+    params = SamplingParams(max_new_tokens=batch + warmup + steps + 8, eos_token_ids=())
+    reqs = [engine.submit([rng.randrange(vocab) for _ in range(context - 1)], sampling=params)
+            for _ in range(batch)]
+    while any(not r.output for r in reqs):          # prefill, a portion per step
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        n = engine.step()
+        assert n == batch, f"a timed step ran {n} tokens, expected {batch}"
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for r in reqs:
+        r.cancelled = True
+    engine.scheduler.retire_finished()
+    return batch * steps / dt, dt / steps * 1e3
+
+
+def prefill_rate(engine, tokens, vocab, seed, repeats=3):
+    """Time one step that runs a whole prompt of ``tokens`` tokens and samples its first token."""
+    import torch
+    from socrates_amd.sampling import SamplingParams
+    rng = random.Random(seed)
+    best = None
+    for _ in range(repeats + 1):
+        req = engine.submit([rng.randrange(vocab) for _ in range(tokens)],
+                            sampling=SamplingParams(max_new_tokens=1, eos_token_ids=()))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n = engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert n == tokens and req.done
+        engine.scheduler.retire_finished()
+        best = dt if best is None else min(best, dt)      # the first repeat warms up
+    return best
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048)
+    ap.add_argument("--max-len", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has")
+    ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is "
+              "single-GPU by design)")
+        return 2
+
+    import torch
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    item = 2 if args.dtype == "bf16" else 4
+    cfg = dict(QWEN3_4B, num_hidden_layers=args.layers)
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
+    V = config.vocab_size
+
+    tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
+    # bytes one decode step has to read: every weight once, and the cache of the live requests
+    step_bytes = (config.param_counts()["read_per_step"] * item
+                  + args.batch * args.context * config.kv_bytes_per_token(item))
+    achieved = step_bytes / (ms * 1e-3) / 1e9
+
+    pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
+    pre_flops = config.prefill_flops(args.prefill_tokens)
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            points[f"decode_b{b}"] = round(decode_rate(engine, b, args.context, max(8, args.steps // 2),
+                                                       4, V, seed=3 + b)[0], 1)
+    out = {
+        "metric": "decode tok/s @ batch 8, context 2048 (Qwen3-4B-sized, bf16)",
+        "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: seeded random weights, uniform random token ids",
+        "config": {"model": "Qwen3-4B-sized", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_full": FULL_LAYERS,
+                   "hidden_size": config.hidden_size, "num_attention_heads": config.num_attention_heads,
+                   "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+                   "intermediate_size": config.intermediate_size, "vocab_size": V,
+                   "tie_word_embeddings": config.tie_word_embeddings, "max_len": args.max_len,
+                   "block_size": 16, "hip_graphs": not args.no_graphs},
+        "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
+                    "ms": round(pre_s * 1e3, 3),
+                    "frac": round(pre_flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+        "points": points,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

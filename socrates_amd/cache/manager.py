@@ -239,6 +239,29 @@ class CacheManager:
             short = max(short, g.missing(row, new_len) - freed - g.allocator.n_free)
         return max(short, 0)
 
+    def pages_needed(self, row: int, new_len: int):
+        """Per group: pages ``row`` would take to grow to ``new_len`` tokens, minus the pages
+        that step would give back first (may be negative)."""
+        self._check_open(row)
+        start = self.length(row)
+        return [g.missing(row, new_len) - (g.droppable(row, start) - g.first_live[row])
+                for g in self.groups]
+
+    def free_pages(self):
+        """Per group: pages free now."""
+        return [g.allocator.n_free for g in self.groups]
+
+    def held_pages(self, row: int):
+        """Per group: pages ``row`` holds now."""
+        return [g.covered[row] - g.first_live[row] for g in self.groups]
+
+    @property
+    def pool_tokens(self) -> int:
+        """Tokens one request can hold if it has the whole pool of every group."""
+        if not self.groups:
+            return self.max_len
+        return min(self.max_len, min(g.allocator.num_blocks for g in self.groups) * self.block_size)
+
     def reserve(self, row: int, new_len: int):
         """Make sure every group holds the pages for positions up to ``new_len`` of
         ``row``, after giving back the pages its next tokens can no longer see.

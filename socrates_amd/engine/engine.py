@@ -1,0 +1,165 @@
+"""The engine: submit, admit, run portions of prompts beside decoding rows, sample,
+finish and free.
+
+The surface follows the reference's ``Engine`` (model/inference_paged.py:54-238):
+the same constructor arguments with the same meanings (``model``, ``tok``,
+``device``, ``dtype``, ``compile``, ``max_batch``, ``max_len``, ``max_new_tokens``,
+``block_size``, ``num_blocks``), ``submit`` returning a ``Request``, ``run`` until
+everything is finished, results in ``req.output``. Differences: ``model`` is a
+model folder (or a ready ``ModelRunner``), a prompt may be a list of token ids (a
+tokenizer is optional), prompts are prefilled in portions of at most ``chunk``
+tokens in the same step as the decoding rows, pages are taken lazily, and
+``generate`` wraps submit + run.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..cache import blocks_for
+from ..sampling import Sampler, SamplingParams
+from .batch import StepEntry
+from .request import MAX_BATCH, MAX_LEN, MAX_NEW_TOKENS, MAX_QUEUE, QueueFull, Request, TooLong  # noqa: F401
+from .runner import ModelRunner
+from .scheduler import Scheduler
+
+KV_BLOCK = 16          # model/inference_paged.py:51
+PREFILL_CHUNK = 2048   # token budget of one step
+
+
+class Engine:
+    def __init__(self, model, tok=None, device: str = "cuda:0", dtype=torch.bfloat16,
+                 compile: bool = True, max_batch: int = MAX_BATCH, max_len: int = MAX_LEN,
+                 max_new_tokens: int = MAX_NEW_TOKENS, block_size: int = KV_BLOCK,
+                 num_blocks: Optional[int] = None, chunk: int = PREFILL_CHUNK,
+                 max_queue: int = MAX_QUEUE):
+        """model: a model folder (config.json + safetensors) or a ModelRunner. tok: an
+        optional tokenizer with the HF surface the reference uses (``apply_chat_template``,
+        ``__call__``, ``all_special_ids``); without one, prompts are token id lists.
+        compile: replay decode-only steps from captured HIP graphs. num_blocks: pages in the
+        pool; default is the worst case max_batch * ceil(max_len / block_size)
+        (model/inference_paged.py:83-84)."""
+        self.device, self.max_batch = device, max_batch
+        self.max_len, self.max_new_tokens = max_len, max_new_tokens
+        self.tok = tok
+        if isinstance(model, ModelRunner):
+            self.runner = model
+        else:
+            per_row = blocks_for(max_len, block_size)
+            self.runner = ModelRunner.from_folder(
+                model, dtype, device, max_rows=max_batch, max_len=max_len, block_size=block_size,
+                num_blocks=num_blocks or max_batch * per_row)
+        self.cache = self.runner.cache
+        self.plan_ = self.runner.model.plan
+        self.scheduler = Scheduler(self.cache, max_batch, max_len, chunk, max_queue)
+        self.sampler = Sampler(self.runner.ops, self.cache.scalars)
+        self.compile = compile
+        if compile and hasattr(self.runner, "enable_graphs"):
+            self.runner.enable_graphs(max_batch)
+        self.n_steps = 0
+        self.prompt_tokens = 0          # counters in place of the reference's Prometheus ones
+        self.output_tokens = 0
+
+    # -- reference-compatible views ------------------------------------------------------------
+    @property
+    def pending(self):
+        return self.scheduler.pending
+
+    @property
+    def rows(self):
+        return self.scheduler.running
+
+    @property
+    def n_active(self) -> int:
+        return len(self.scheduler.running)
+
+    # -- submitting ------------------------------------------------------------------------------
+    def submit(self, prompt, stream: bool = False, sampling: Optional[SamplingParams] = None) -> Request:
+        """Queue a prompt (text if the engine has a tokenizer, else token ids). Raises
+        QueueFull or TooLong as the reference does (model/inference_paged.py:132-148)."""
+        sampling = sampling or SamplingParams()
+        if isinstance(prompt, str):
+            if self.tok is None:
+                raise ValueError("a text prompt needs a tokenizer; pass token ids instead")
+            text = self.tok.apply_chat_template(
+                [{"role": "user", "content": prompt}], tokenize=False, add_generation_prompt=True,
+                enable_thinking=False)
+            ids = self.tok(text, return_tensors="pt").input_ids
+            ids = [int(t) for t in (ids[0].tolist() if hasattr(ids, "shape") else ids[0])]
+        else:
+            ids = [int(t) for t in prompt]
+        eos = sampling.eos_token_ids
+        if eos is None:
+            eos = tuple(self.tok.all_special_ids) if self.tok is not None else self.plan_.eos_token_ids
+        req = Request(prompt=prompt, ids=ids, sampling=sampling, eos_token_ids=tuple(eos),
+                      max_new_tokens=(sampling.max_new_tokens if sampling.max_new_tokens is not None
+                                      else self.max_new_tokens))
+        if stream:
+            import queue
+            req.stream = queue.Queue()
+        if any(t < 0 or t >= self.plan_.vocab_size for t in ids):
+            raise ValueError(f"token ids must lie in [0, {self.plan_.vocab_size})")
+        self.scheduler.submit(req)
+        return req
+
+    # -- one step --------------------------------------------------------------------------------
+    def step(self) -> int:
+        """Plan and run one step. Returns the number of tokens it ran (0: nothing to do)."""
+        plan = self.scheduler.plan()
+        if not plan:
+            return 0
+        entries = [StepEntry(p.request.row, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
+                   for p in plan]
+        logits = self.runner.step(entries)
+        wanted = [p for p in plan if p.wants_logits]
+        tokens = self.sampler.sample(logits, [p.request.row for p in wanted])
+        for p in plan:
+            if not p.request.output:
+                self.prompt_tokens += len(p.tokens)
+        for p, token in zip(wanted, tokens):
+            self.record(p.request, token)
+        self.n_steps += 1
+        return sum(len(p.tokens) for p in plan)
+
+    def record(self, req: Request, token: int) -> None:
+        """A stop token ends the request and is not kept (model/inference_paged.py:200-211);
+        the request also ends when ``max_new_tokens`` tokens are kept, without running a
+        further step for a token that would be dropped."""
+        now = time.perf_counter()
+        if not req.first_token:
+            req.first_token = now
+        if token in req.eos_token_ids:
+            req.done = True
+        else:
+            req.output.append(token)
+            self.output_tokens += 1
+            if req.stream is not None:
+                req.stream.put(token)
+            if len(req.output) >= req.max_new_tokens:
+                req.done = True
+        if req.done:
+            req.finished = now
+            if req.stream is not None:
+                req.stream.put(None)
+
+    def run(self) -> None:
+        """Until nothing is pending or running (model/inference_paged.py:231-237)."""
+        while not self.scheduler.idle:
+            if self.step() == 0 and not self.scheduler.idle:
+                raise RuntimeError("requests are waiting but nothing can be scheduled")
+
+    # -- the Python entry point ------------------------------------------------------------------
+    def generate(self, prompts: Sequence, max_new_tokens: Optional[int] = None,
+                 temperature: float = 0.0, seed: int = 0,
+                 eos_token_ids: Optional[Sequence[int]] = None) -> List[List[int]]:
+        """Generate for every prompt; returns the new token ids of each. Request i draws
+        from the random stream ``seed + i``."""
+        reqs = [self.submit(p, sampling=SamplingParams(
+            temperature=temperature, seed=seed + i, max_new_tokens=max_new_tokens,
+            eos_token_ids=None if eos_token_ids is None else tuple(eos_token_ids)))
+            for i, p in enumerate(prompts)]
+        self.run()
+        return [r.output for r in reqs]
