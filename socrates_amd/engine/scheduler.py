@@ -16,8 +16,9 @@ that pages run out is decided as follows:
   cache is recomputed later as a prompt portion). If none is younger, a prompt
   portion is shortened to what fits, and otherwise the request waits; the oldest
   request always fits, because ``submit`` refuses what the whole pool cannot hold.
-* New requests are admitted in arrival order while a row, budget and pages for
-  at least one token are free, and only if no running request had to wait.
+* New requests are admitted in arrival order while a row and budget are free and the
+  pool has pages for all tokens the request has so far plus one, and only if no
+  running request had to wait or was preempted in this step.
 """
 
 from __future__ import annotations
@@ -119,6 +120,11 @@ class Scheduler:
         """Retire what is finished, then choose the next step's entries. Preempts and
         admits as a side effect. An empty plan means there is nothing to run."""
         self.retire_finished()
+        if any(r.cancelled for r in self.pending):
+            for r in self.pending:
+                if r.cancelled:
+                    r.event.set()
+            self.pending = deque(r for r in self.pending if not r.cancelled)
         cache = self.cache
         plan: List[Planned] = []
         budget = self.token_budget
@@ -165,8 +171,13 @@ class Scheduler:
             todo = req.tokens()
             row = cache.open_row()
             n = min(len(todo), budget)
-            if not self._fits(cache.pages_needed(row, n), free):
-                n = self._longest_fit(row, 0, n, free)
+            # Pages for everything the request has so far, and its next token, must be free
+            # (else it would soon take pages from, or be preempted by, the running ones).
+            if not self._fits(cache.pages_needed(row, len(todo) + 1), free):
+                if self.running:
+                    cache.close_row(row)
+                    break
+                n = self._longest_fit(row, 0, n, free)      # alone: the pool is as free as it gets
             if n == 0:
                 cache.close_row(row)
                 break

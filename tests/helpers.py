@@ -23,12 +23,13 @@ TINY_B = dict(cfg=dict(architectures=["Qwen3ForCausalLM"], vocab_size=384, hidde
                        head_dim=32, intermediate_size=160, rms_norm_eps=1e-5, rope_theta=1e6,
                        tie_word_embeddings=False),
               block_size=8, gain_std=0.2)
-# A third one with awkward sizes: three query heads per group, head size 48, odd widths.
+# A third one with awkward sizes: three kv heads with three query heads each, head size 48,
+# odd widths. It differs from A and from B in every size and option.
 TINY_C = dict(cfg=dict(architectures=["Qwen3ForCausalLM"], vocab_size=331, hidden_size=72,
-                       num_hidden_layers=2, num_attention_heads=6, num_key_value_heads=2,
+                       num_hidden_layers=4, num_attention_heads=9, num_key_value_heads=3,
                        head_dim=48, intermediate_size=200, rms_norm_eps=3e-6, rope_theta=50000.0,
-                       tie_word_embeddings=False),
-              block_size=16, gain_std=0.1)
+                       tie_word_embeddings=True),
+              block_size=4, gain_std=0.1)
 
 TINIES = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 

@@ -362,3 +362,28 @@ def test_sampling(kernel_sets):
     # temperature to zero converges to argmax
     cold = hip.sample(lg, torch.full((n,), 1e-4, device=DEV), seed, draws)
     assert cold.tolist() == lg.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("far", [0, 3, 15, 16, 17, 255, 256, 511])
+def test_attention_far_key_stands_out(kernel_sets, dtype, far):
+    """Among 700 near-uniform keys one far key matches the query strongly, so it takes almost
+    all the weight: a kernel that skips it, or reads a neighbour instead (a page edge, a
+    split seam), returns another value row by O(1), which random keys would hide."""
+    hip, _ = kernel_sets[dtype]
+    Hq, Hkv, D, bs, n = 8, 2, 64, 16, 700
+    slot, dense = make_paged_case([n], Hq, Hkv, D, bs, dtype, seed=far + 1)
+    u = torch.nn.functional.normalize(torch.randn(D), dim=0)
+    q = (0.1 * torch.randn(1, Hq, D) + 6.0 * u).to(dtype).to(DEV)
+    page, off = int(slot.block_table[0, far // bs]), far % bs
+    slot.k[page, :, off] = (6.0 * u).to(dtype).to(DEV)
+    slot.v[page, :, off] = torch.arange(D, dtype=torch.float32).to(dtype).to(DEV) / 8
+    dense[0][0][:, far] = slot.k[page, :, off].float().cpu()
+    dense[0][1][:, far] = slot.v[page, :, off].float().cpu()
+    want = dense_attention(q, dense, [0], [n - 1], 1.0)
+    assert (want.view(Hq, D) - slot.v[page, 0, off].float().cpu()).abs().max() < 0.05    # the far key dominates
+    for splits in (None, (128, 6), (1 << 30, 1)):
+        hip.attention_splits = splits
+        got = hip.paged_attention(q, slot, ctx_for([0], [n - 1]), 1.0)
+        close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 3e-2)
+    hip.attention_splits = None

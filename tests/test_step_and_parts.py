@@ -1,0 +1,293 @@
+"""The step function, each part alone, and the generality of the layer recipe.
+
+Every test runs with the torch stand-in for the kernels on the CPU (``not gpu``) and with
+the HIP kernels in float32 and bfloat16 on the GPU (``gpu``)."""
+
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import (TINIES, TINY_B, make_runner, random_prompts, replay, trace_mixed, trace_portions,
+                     trace_tail_decode, trace_whole, write_tiny)
+from socrates_amd.cache import CacheManager
+from socrates_amd.config import AttentionSpec, BlockSpec, ModelPlan, Qwen3Config, RMSNormSpec, RopeSpec, RunStep, SwiGLUSpec
+from socrates_amd.engine import ModelRunner, StepEntry, build_context
+from socrates_amd.parts import (DecoderModel, RowState, TensorDecl, build_block, build_part, cache_needs,
+                                expected_tensors, register_part)
+from socrates_amd.weights import random_tensors
+
+KINDS = [pytest.param("torch", torch.float32, id="cpu-fp32"),
+         pytest.param("hip", torch.float32, id="gpu-fp32", marks=pytest.mark.gpu),
+         pytest.param("hip", torch.bfloat16, id="gpu-bf16", marks=pytest.mark.gpu)]
+TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
+
+
+def kernels(kind, dtype):
+    if kind == "torch":
+        from torch_kernels import TorchKernels
+        return TorchKernels(dtype, "cpu")
+    from socrates_amd.kernels import HipKernels
+    return HipKernels(dtype, "cuda:0")
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("parts_models")
+    return {name: write_tiny(base / name, tiny, seed=20 + i) for i, (name, tiny) in enumerate(TINIES.items())}
+
+
+@pytest.mark.parametrize("name", list(TINIES))
+def test_every_cut_equals_the_plain_forward_on_the_cpu(folders, name):
+    cfg, w = plain.read_folder(folders[name])
+    prompts = random_prompts([5, 17, 33, 70], cfg["vocab_size"], seed=0)
+    want = {f"r{i}": plain.forward(cfg, w, p) for i, p in enumerate(prompts)}
+    from torch_kernels import TorchKernels
+    for steps in (trace_whole(prompts), trace_tail_decode(prompts, 32), trace_portions(prompts, 1),
+                  trace_mixed(prompts, 2)):
+        runner = make_runner(folders[name], TorchKernels(torch.float32, "cpu"), max_rows=4, max_len=128,
+                             block_size=TINIES[name]["block_size"], num_blocks=160 // TINIES[name]["block_size"])
+        got = replay(runner, steps)
+        for rid in want:
+            torch.testing.assert_close(got[rid], want[rid], atol=2e-5, rtol=2e-5)
+
+
+def ctx_of(ops, lens, starts=None, rows=None):
+    starts = starts or [0] * len(lens)
+    rows = rows if rows is not None else list(range(len(lens)))
+    entries = [StepEntry(r, [0] * n, []) for r, n in zip(rows, lens)]
+    return build_context(entries, starts, ops.device)
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_each_part_alone(folders, kind, dtype):
+    """Norm, rotation, attention mixer, feed-forward and block, each built from its spec and
+    tensors alone, against the plain function of the same part."""
+    ops = kernels(kind, dtype)
+    cfg, w = plain.read_folder(folders["B"])
+    config = Qwen3Config.from_dict(TINY_B["cfg"])
+    plan = config.plan()
+    spec = plan.layers[1]
+    dev = lambda t, dt=dtype: t.to(dt).to(ops.device).clone()
+    T = 19
+    x = torch.randn(T, config.hidden_size) * 0.5
+    tol = TOL[dtype]
+
+    norm = build_part(spec.norm1, {"weight": dev(w["model.layers.1.input_layernorm.weight"], torch.float32)}, ops)
+    residual = dev(x, torch.float32)
+    got = norm.add_norm(residual, None)
+    x_used = x.to(torch.float32)
+    torch.testing.assert_close(got.float().cpu(), plain.rms_norm(x_used, w["model.layers.1.input_layernorm.weight"],
+                                                                 cfg["rms_norm_eps"]), **tol)
+
+    rope = build_part(spec.mixer.position, {}, ops)
+    q = torch.randn(T, 8, 32)
+    k = torch.randn(T, 2, 32)
+    qd, kd = dev(q), dev(k)
+    positions = torch.arange(3, 3 + T, dtype=torch.int32, device=ops.device)
+    rope.apply(qd, kd, positions)
+    cos, sin = plain.rope_angles(32, cfg["rope_theta"], torch.arange(3, 3 + T))
+    torch.testing.assert_close(qd.float().cpu(), plain.apply_rope(q.to(dtype).float(), cos, sin), **tol)
+    torch.testing.assert_close(kd.float().cpu(), plain.apply_rope(k.to(dtype).float(), cos, sin), **tol)
+
+    p = "model.layers.1."
+    ffn = build_part(spec.ffn, {n: dev(w[p + "mlp." + n]) for n in ("gate_proj.weight", "up_proj.weight",
+                                                                     "down_proj.weight")}, ops)
+    xin = dev(x)
+    torch.testing.assert_close(ffn.forward(xin).float().cpu(), plain.swiglu_mlp(xin.float().cpu(), w, p + "mlp."), **tol)
+
+    att_tensors = {n: dev(w[p + "self_attn." + n], torch.float32 if "norm" in n else dtype)
+                   for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight",
+                             "q_norm.weight", "k_norm.weight")}
+    mixer = build_part(spec.mixer, att_tensors, ops)
+    cache = CacheManager([type(mixer).cache_need(spec.mixer)], 2, 64, 8, 12, dtype, ops.device)
+    row = cache.open_row()
+    cache.reserve(row, T)
+    cache.sync()
+    ctx = ctx_of(ops, [T])
+    got = mixer.forward(xin, ctx, cache.slot(0), True)
+    want = plain.attention_layer(xin.float().cpu(), w, p + "self_attn.", cfg, torch.arange(T))
+    torch.testing.assert_close(got.float().cpu(), want, **tol)
+
+    block_w = {n: dev(t, torch.float32 if t.dim() == 1 else dtype) for n, t in w.items() if n.startswith(p)}
+    block = build_block(spec, block_w, ops)
+    cache = CacheManager([type(mixer).cache_need(spec.mixer)], 2, 64, 8, 12, dtype, ops.device)
+    cache.reserve(cache.open_row(), T)
+    cache.sync()
+    residual = dev(x, torch.float32)
+    pending = block.forward(residual, None, ctx, cache.slot(0), True)
+    torch.testing.assert_close(residual.cpu() + pending.float().cpu(), plain.block(x, w, 1, cfg, torch.arange(T)), **tol)
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_attention_part_with_a_window_in_portions(kind, dtype):
+    """The attention part with window 5 over a cache group that gives pages back, fed in
+    portions; one key and query are scaled so that the score at the window's edge stands
+    out: reading one key too many or too few changes the output by O(1)."""
+    ops = kernels(kind, dtype)
+    Hq, Hkv, D, hidden, W, T = 4, 2, 16, 32, 5, 41
+    spec = AttentionSpec(hidden, Hq, Hkv, D, scale=D ** -0.5, qk_norm=None, position=None, window=W)
+    g = torch.Generator().manual_seed(5)
+    wq, wk, wv, wo = (torch.randn(s, generator=g) * 0.3 for s in ((Hq * D, hidden), (Hkv * D, hidden),
+                                                                  (Hkv * D, hidden), (hidden, Hq * D)))
+    x = torch.randn(T, hidden, generator=g)
+    x[20] *= 6.0            # key 20 stands out for every later query that still sees it
+    dev = lambda t: t.to(dtype).to(ops.device)
+    mixer = build_part(spec, {"q_proj.weight": dev(wq), "k_proj.weight": dev(wk), "v_proj.weight": dev(wv),
+                              "o_proj.weight": dev(wo)}, ops)
+    xr = x.to(dtype).float()
+    q = (xr @ wq.to(dtype).float().T).view(T, Hq, D)
+    k = (xr @ wk.to(dtype).float().T).view(T, Hkv, D)
+    v = (xr @ wv.to(dtype).float().T).view(T, Hkv, D)
+    if dtype == torch.bfloat16:
+        q, k, v = (t.to(dtype).float() for t in (q, k, v))
+    want = plain.attention_scores(q, k, v, D ** -0.5, window=W).reshape(T, Hq * D) @ wo.to(dtype).float().T
+    cache = CacheManager([type(mixer).cache_need(spec)], 2, 64, 4, 6, dtype, ops.device)   # 6 pages of 4
+    row = cache.open_row()
+    outs, t = [], 0
+    for n in (3, 1, 7, 2, 1, 1, 9, 4, 13):
+        cache.reserve(row, t + n)
+        cache.sync()
+        ctx = ctx_of(ops, [n], [t], [row])
+        outs.append(mixer.forward(dev(x[t:t + n]), ctx, cache.slot(0), True).float().cpu())
+        cache.advance(row, n)
+        cache.check()
+        t += n
+    # 41 tokens are 11 pages of 4; the pool has 6: pages behind the window were given back
+    assert t == T and cache.held_pages(row)[0] <= 5 and cache.groups[0].first_live[row] == 6
+    tol = dict(atol=2e-4, rtol=2e-4) if dtype == torch.float32 else dict(atol=0.25, rtol=5e-2)
+    torch.testing.assert_close(torch.cat(outs), want, **tol)
+    off_by_one = plain.attention_scores(q, k, v, D ** -0.5, window=W + 1).reshape(T, Hq * D) @ wo.to(dtype).float().T
+    assert (off_by_one - want).abs().max() > 1.0              # the test can tell the edge
+
+
+def plan_with(layers, order, hidden, vocab=50):
+    return ModelPlan(architecture="Toy", vocab_size=vocab, hidden=hidden, layers=tuple(layers), order=tuple(order),
+                     final_norm=RMSNormSpec(hidden, 1e-6), embedding_name="embed.weight",
+                     final_norm_prefix="final_norm", head_name=None)
+
+
+def qwen_like_block(i, hidden=32, heads=4, kv=2, D=16, ff=48, theta=1e4, eps=1e-6):
+    att = AttentionSpec(hidden, heads, kv, D, D ** -0.5, RMSNormSpec(D, eps), RopeSpec(D, theta))
+    return BlockSpec(att, SwiGLUSpec(hidden, ff), RMSNormSpec(hidden, eps), RMSNormSpec(hidden, eps),
+                     prefix=f"model.layers.{i}.")
+
+
+def run_whole_and_cut(plan, ops, tokens, cuts, max_len=64, bs=8):
+    weights = random_tensors(expected_tensors(plan), seed=3, dtype=ops.dtype, device=ops.device, std=0.2, gain_std=0.1)
+    out = []
+    for cut in cuts:
+        model = DecoderModel(plan, weights, ops)
+        cache = CacheManager(cache_needs(plan), 2, max_len, bs, 2 * max_len // bs, ops.dtype, ops.device)
+        runner = ModelRunner(model, cache)
+        row = cache.open_row()
+        logits, t = [], 0
+        for n in cut:
+            logits.append(runner.step([StepEntry(row, tokens[t:t + n], list(range(n)))]).float().cpu())
+            t += n
+        out.append(torch.cat(logits))
+    return weights, out
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_a_layer_may_run_twice_and_read_another_runs_cache(kind, dtype):
+    """Run order as data: layer 1 appears twice; its second run reads the keys and values
+    its first run stored (it stores none itself). Checked against the plain functions put
+    together the same way, whole and in portions."""
+    ops = kernels(kind, dtype)
+    layers = [qwen_like_block(0), qwen_like_block(1)]
+    order = [RunStep(0, 0), RunStep(1, 1), RunStep(1, 1, write=False)]
+    plan = plan_with(layers, order, hidden=32)
+    tokens = random_prompts([23], 50, seed=4)[0]
+    weights, (whole, cut) = run_whole_and_cut(plan, ops, tokens, [[23], [5, 1, 9, 2, 6]])
+    w = {n: t.float().cpu() for n, t in weights.items()}
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6, rope_theta=1e4)
+    pos = torch.arange(23)
+    x = w["embed.weight"][torch.tensor(tokens)]
+    x = plain.block(x, w, 0, cfg, pos)
+    h1 = plain.rms_norm(x, w["model.layers.1.input_layernorm.weight"], 1e-6)
+    x = plain.block(x, w, 1, cfg, pos)
+    # second run of layer 1: queries from the new input, keys and values from the first run
+    p = "model.layers.1.self_attn."
+    h2 = plain.rms_norm(x, w["model.layers.1.input_layernorm.weight"], 1e-6)
+    cos, sin = plain.rope_angles(16, 1e4, pos)
+    q = plain.apply_rope(plain.rms_norm((h2 @ w[p + "q_proj.weight"].T).view(23, 4, 16), w[p + "q_norm.weight"], 1e-6), cos, sin)
+    k = plain.apply_rope(plain.rms_norm((h1 @ w[p + "k_proj.weight"].T).view(23, 2, 16), w[p + "k_norm.weight"], 1e-6), cos, sin)
+    v = (h1 @ w[p + "v_proj.weight"].T).view(23, 2, 16)
+    x = x + plain.attention_scores(q, k, v, 0.25).reshape(23, 64) @ w[p + "o_proj.weight"].T
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["model.layers.1.post_attention_layernorm.weight"], 1e-6), w, "model.layers.1.mlp.")
+    want = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
+    tol = TOL[dtype] if dtype == torch.float32 else dict(atol=0.15, rtol=5e-2)
+    torch.testing.assert_close(whole, want, **tol)
+    torch.testing.assert_close(cut, want, **tol)
+
+
+# ---- a toy mixer with a state of its own, defined here and registered from outside ------------
+@dataclass(frozen=True)
+class DecaySpec:
+    """y_t = W s_t with s_t = decay * s_{t-1} + x_t: a running, decaying sum per request."""
+    hidden: int
+    decay: float
+
+
+class DecayMixer:
+    @staticmethod
+    def tensors(spec):
+        return {"mix.weight": TensorDecl((spec.hidden, spec.hidden))}
+
+    @staticmethod
+    def cache_need(spec):
+        return RowState((spec.hidden,))
+
+    def __init__(self, spec, tensors, ops):
+        self.spec, self.ops, self.w = spec, ops, tensors["mix.weight"]
+
+    def forward(self, x, ctx, slot, write=True):
+        starts, rows = ctx.host["seq_qstart"], ctx.host["seq_rows"]
+        states = torch.empty((x.shape[0], self.spec.hidden), dtype=torch.float32, device=x.device)
+        for i, row in enumerate(rows):                       # strictly in position order per request
+            s = slot.state[int(row)]
+            for t in range(int(starts[i]), int(starts[i + 1])):
+                s = self.spec.decay * s + x[t].float()
+                states[t] = s
+            if write:
+                slot.state[int(row)] = s
+        return self.ops.linear(states.to(self.ops.dtype), self.w)
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_a_toy_mixer_with_state_registers_builds_and_steps(kind, dtype):
+    """No file of the framework changes: the spec and the class are registered here; the cache
+    manager gives the mixer a fixed-size state per request, cleared when a row opens."""
+    register_part(DecaySpec, DecayMixer)
+    ops = kernels(kind, dtype)
+    hidden = 32
+    toy = BlockSpec(DecaySpec(hidden, 0.9), SwiGLUSpec(hidden, 40), RMSNormSpec(hidden, 1e-5),
+                    RMSNormSpec(hidden, 1e-5), prefix="model.layers.1.",
+                    names=(("norm1", "n1"), ("mixer", "decay"), ("norm2", "n2"), ("ffn", "mlp")))
+    plan = plan_with([qwen_like_block(0), toy, qwen_like_block(2, heads=2, kv=1)],
+                     [RunStep(0, 0), RunStep(1, 1), RunStep(2, 2)], hidden)
+    assert "model.layers.1.decay.mix.weight" in expected_tensors(plan)
+    needs = cache_needs(plan)
+    assert isinstance(needs[1], RowState) and needs[0] != needs[2]          # two paged groups and a state
+    tokens = random_prompts([21], 50, seed=6)[0]
+    weights, (whole, cut, other) = run_whole_and_cut(plan, ops, tokens, [[21], [4, 1, 1, 8, 2, 5], [20, 1]])
+    tol = dict(atol=2e-4, rtol=2e-4) if dtype == torch.float32 else dict(atol=0.2, rtol=5e-2)
+    torch.testing.assert_close(cut, whole, **tol)
+    torch.testing.assert_close(other, whole, **tol)
+    # a plain recurrence for the toy layer alone confirms the state semantics
+    w = {n: t.float().cpu() for n, t in weights.items()}
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6, rope_theta=1e4)
+    x = plain.block(w["embed.weight"][torch.tensor(tokens)], w, 0, cfg, torch.arange(21))
+    h = plain.rms_norm(x, w["model.layers.1.n1.weight"], 1e-5)
+    s, ys = torch.zeros(hidden), []
+    for t in range(21):
+        s = 0.9 * s + h[t]
+        ys.append(s @ w["model.layers.1.decay.mix.weight"].T)
+    x = x + torch.stack(ys)
+    x = x + plain.swiglu_mlp(plain.rms_norm(x, w["model.layers.1.n2.weight"], 1e-5), w, "model.layers.1.mlp.")
+    cfg2 = dict(cfg, num_attention_heads=2, num_key_value_heads=1)
+    x = plain.block(x, w, 2, cfg2, torch.arange(21))
+    want = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
+    torch.testing.assert_close(whole, want, **tol)
