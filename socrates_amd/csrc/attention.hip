@@ -257,4 +257,307 @@ SOC_EXPORT int soc_paged_attention_tokens(const void* q, const void* k_pool, con
                                 n_splits, stream);
 }
 
+
+// =============================================================================================
+// MFMA path (bfloat16). One wave owns a block of rows that share a cache row and a kv head:
+// rows are (token, query head of the group) pairs, 16 per row tile, RT row tiles per wave.
+// A single decoded token fills G of the 16 rows; a prompt portion fills all of them with
+// consecutive tokens. The wave walks the keys of its split 16 at a time:
+//   S^T[key, row]  = K_tile [16 x D] * Q^T [D x 16]        (A = keys, B = rows)
+//   online softmax per row: a row is an MFMA column, so its running maximum, its scale and
+//   its sum live in the lanes of that column; the maximum over the 16 keys of a tile
+//   needs two cross-lane steps
+//   O^T[d, row]   += V_tile^T [16 d x 16 keys] * P^T [16 keys x 16 rows]
+// S^T comes out of the first product in exactly the lane layout the second one wants for
+// its B operand, so P never leaves registers. V pages are row-major [slot][d]; the V tile
+// is staged through LDS (wave-private) to read it transposed. Scores, softmax and both
+// accumulators are float32; P is rounded to bfloat16 for the second product, as V is.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+constexpr bool QK_K32 = (D % 32 == 0);
+constexpr int QK_STEPS = QK_K32 ? D / 32 : D / 16;
+constexpr int DV = D / 16;                   // 16-wide blocks of the head dimension
+constexpr int V_STRIDE = D + 4;              // LDS row stride (elements): conflict-free transposed reads
+constexpr int V_CHUNKS = 16 * D / 8;         // 16-byte chunks in a 16-key V tile
+constexpr int V_PER_LANE = (V_CHUNKS + 63) / 64;
+
+struct KFrag { uint4 v[QK_STEPS]; };         // K32: 16 bytes per step; K16: the low 8 bytes
+
+__device__ __forceinline__ f32x4_t qk_mfma(const uint4& a, const uint4& b, f32x4_t c) {
+    if constexpr (QK_K32) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(&a),
+                                                       *reinterpret_cast<const bf16x8_t*>(&b), c, 0, 0, 0);
+    } else {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s16x4_t*>(&a),
+                                                         *reinterpret_cast<const s16x4_t*>(&b), c, 0, 0, 0);
+    }
+}
+
+// The slice of a K (or Q) row that this lane feeds to QK step `kk`.
+__device__ __forceinline__ uint4 load_qk_slice(const bf16* row, int kk, int kb) {
+    if constexpr (QK_K32) {
+        return *reinterpret_cast<const uint4*>(row + kk * 32 + kb * 8);
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2*>(row + kk * 16 + kb * 4);
+        return make_uint4(t.x, t.y, 0u, 0u);
+    }
+}
+
+template <int RT>
+__global__ void __launch_bounds__(256)
+paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
+                       const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
+                       int table_width, const int* __restrict__ token_rows,
+                       const int* __restrict__ positions, const int* __restrict__ row_blocks,
+                       int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
+                       float* __restrict__ part_ml, int Hq, int Hkv, int BS, float scale, int window,
+                       int split_len, int n_splits, int group_pad_log2) {
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[4][16 * V_STRIDE];
+    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    const int G = Hq / Hkv;
+    const int Gp = 1 << group_pad_log2;                 // rows per token in a row block
+    const int chunks = (G + 15) / 16;                   // head chunks when G > 16
+    const int task = blockIdx.x * 4 + wave;
+    if (task >= n_row_blocks * Hkv * chunks) return;
+    const int blk = task / (Hkv * chunks);
+    const int kvh = (task / chunks) % Hkv, chunk = task % chunks;
+    const int split = blockIdx.y;
+    const int tok0 = row_blocks[2 * blk], ntok = row_blocks[2 * blk + 1];
+    const int pos0 = positions[tok0];
+    const int* table = block_table + (size_t)token_rows[tok0] * table_width;
+
+    // keys this wave walks: its split, cut to what its rows can see
+    int klo = split * split_len;
+    int khi = min(klo + split_len, pos0 + ntok);
+    if (window > 0) klo = max(klo, pos0 - window + 1);
+    const int kmin = klo;                                // first key any row of the block can see
+    klo = klo & ~15;                                     // tiles are aligned to 16 keys
+    const int li = lane % 16, kb = lane / 16;
+    uint16_t* vl = v_lds[wave];
+
+    // rows of this lane's column, per row tile
+    int row_pos[RT];                                     // position of the row's token, -1: no row
+    size_t row_q[RT];                                    // offset of the row's query / output
+    uint4 qf[RT][QK_STEPS];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int rho = rt * 16 + li;
+        const int tt = rho >> group_pad_log2, g = chunk * 16 + (rho & (Gp - 1));
+        const bool ok = tt < ntok && g < G;
+        row_pos[rt] = ok ? pos0 + tt : -1;
+        row_q[rt] = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? g : 0)) * D;
+#pragma unroll
+        for (int kk = 0; kk < QK_STEPS; ++kk)
+            qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
+    }
+
+    f32x4_t o[RT][DV];
+    float m[RT], l[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m[rt] = -INFINITY; l[rt] = 0.f;
+#pragma unroll
+        for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    }
+
+    // Global loads of one tile: this lane's K slices and its share of the V tile. Keys that no
+    // row of the block can see are not read at all: zeros stand in for them, so that whatever
+    // lies in stale slots or in the null page (inf, NaN) never meets a product.
+    auto fetch = [&](int key0, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
+        const int key = key0 + li;
+        if (key >= kmin && key < khi) {
+            const int page = table[key / BS];
+            const bf16* krow = k_pool + ((size_t)page * Hkv * BS + (size_t)kvh * BS + key % BS) * D;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int j = 0; j < V_PER_LANE; ++j) {
+            const int c = lane + 64 * j;
+            if (V_CHUNKS % 64 == 0 || c < V_CHUNKS) {
+                const int vk = c / (D / 8), part = c % (D / 8);
+                const int vkey = key0 + vk;
+                if (vkey >= kmin && vkey < khi)
+                    vr[j] = *reinterpret_cast<const uint4*>(
+                        v_pool + ((size_t)table[vkey / BS] * Hkv * BS + (size_t)kvh * BS + vkey % BS) * D + part * 8);
+                else
+                    vr[j] = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    };
+
+    KFrag kf_cur, kf_next;
+    uint4 vr_cur[V_PER_LANE], vr_next[V_PER_LANE];
+    if (klo < khi) fetch(klo, kf_cur, vr_cur);
+    for (int key0 = klo; key0 < khi; key0 += 16) {
+        const bool more = key0 + 16 < khi;
+        if (more) fetch(key0 + 16, kf_next, vr_next);
+        // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk)
+#pragma unroll
+        for (int j = 0; j < V_PER_LANE; ++j) {
+            const int c = lane + 64 * j;
+            if (V_CHUNKS % 64 == 0 || c < V_CHUNKS) {
+                const int vk = c / (D / 8), part = c % (D / 8);
+                uint2* dst = reinterpret_cast<uint2*>(&vl[vk * V_STRIDE + part * 8]);
+                dst[0] = make_uint2(vr_cur[j].x, vr_cur[j].y);
+                dst[1] = make_uint2(vr_cur[j].z, vr_cur[j].w);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        // scores and softmax per row tile
+        s16x4_t pf[RT];
+        bool any_rescale = false;
+        float alpha[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) s = qk_mfma(kf_cur.v[kk], qf[rt][kk], s);
+            float sv[4];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = key0 + 4 * kb + r;
+                bool seen = key <= row_pos[rt] && key < khi && key >= split * split_len;
+                if (window > 0) seen = seen && key > row_pos[rt] - window;
+                sv[r] = seen ? s[r] * scale : -INFINITY;
+                mx = fmaxf(mx, sv[r]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
+            const float mn = fmaxf(m[rt], mx);
+            const float ms = mn == -INFINITY ? 0.f : mn;
+            alpha[rt] = __expf(m[rt] - ms);
+            float psum = 0.f;
+            uint16_t pb[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = __expf(sv[r] - ms);
+                psum += p;
+                pb[r] = f32_to_bf16_bits(p);
+            }
+            l[rt] = l[rt] * alpha[rt] + psum;
+            any_rescale = any_rescale || (m[rt] != mn);
+            m[rt] = mn;
+            pf[rt] = (s16x4_t){(short)pb[0], (short)pb[1], (short)pb[2], (short)pb[3]};
+        }
+        if (__any(any_rescale)) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
+        }
+        // O^T += V^T P^T, one 16-wide block of d at a time; the V^T slice is shared by the row tiles
+#pragma unroll
+        for (int j = 0; j < DV; ++j) {
+            const uint16_t* src = &vl[(4 * kb) * V_STRIDE + j * 16 + li];
+            const s16x4_t vt = (s16x4_t){(short)src[0], (short)src[V_STRIDE], (short)src[2 * V_STRIDE],
+                                         (short)src[3 * V_STRIDE]};
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pf[rt], o[rt][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (more) {
+            kf_cur = kf_next;
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) vr_cur[j] = vr_next[j];
+        }
+    }
+
+    // finish: the row sum is spread over the four lanes of the row's column
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float L = l[rt];
+        L += __shfl_xor(L, 16, SOC_WAVE);
+        L += __shfl_xor(L, 32, SOC_WAVE);
+        if (row_pos[rt] < 0) continue;
+        const size_t base = row_q[rt];                                   // (token * Hq + head) * D
+        if (n_splits == 1) {
+            const float inv = L > 0.f ? 1.0f / L : 0.f;
+#pragma unroll
+            for (int j = 0; j < DV; ++j) {
+                uint2 pk;
+                pk.x = (uint32_t)f32_to_bf16_bits(o[rt][j][0] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][1] * inv) << 16);
+                pk.y = (uint32_t)f32_to_bf16_bits(o[rt][j][2] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][3] * inv) << 16);
+                *reinterpret_cast<uint2*>(out + base + j * 16 + 4 * kb) = pk;
+            }
+        } else {
+            const size_t pi = (base / D) * n_splits + split;
+#pragma unroll
+            for (int j = 0; j < DV; ++j)
+                *reinterpret_cast<float4*>(part_o + pi * D + j * 16 + 4 * kb) =
+                    make_float4(o[rt][j][0], o[rt][j][1], o[rt][j][2], o[rt][j][3]);
+            if (kb == 0) { part_ml[pi * 2] = m[rt]; part_ml[pi * 2 + 1] = L; }
+        }
+    }
+}
+
+// Merge all n_splits partials of a (token, head); an empty split has m = -inf.
+__global__ void paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                        bf16* __restrict__ out, int Hq, int n_splits) {
+    const int h = blockIdx.x, n = blockIdx.y;
+    const size_t base = ((size_t)n * Hq + h) * n_splits;
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = part_ml[(base + s) * 2];
+        if (ms != -INFINITY) L += part_ml[(base + s) * 2 + 1] * __expf(ms - M);
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int e = threadIdx.x; e < D; e += blockDim.x) {
+        float A = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float ms = part_ml[(base + s) * 2];
+            if (ms != -INFINITY) A += part_o[(base + s) * D + e] * __expf(ms - M);
+        }
+        out[((size_t)n * Hq + h) * D + e] = from_float<bf16>(A * inv);
+    }
+}
+
+// bfloat16 only. row_blocks [n_row_blocks, 2] = (first token, tokens) of each block of at most
+// (16 * row_tiles) >> group_pad_log2 tokens of one sequence; 2^group_pad_log2 >= min(G, 16).
+// Splits are over absolute key indices: split s covers keys [s * split_len, (s + 1) * split_len),
+// split_len a multiple of 16; n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml
+// [N, Hq, n_splits, 2], which are written for every (row, split), empty ones with m = -inf.
+SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const void* v_pool,
+                                        const int* block_table, int table_width, const int* token_rows,
+                                        const int* positions, const int* row_blocks, int n_row_blocks,
+                                        void* out, float* part_o, float* part_ml, int N, int Hq, int Hkv,
+                                        int BS, float scale, int window, int split_len, int n_splits,
+                                        int row_tiles, int group_pad_log2, hipStream_t stream) {
+    if (N <= 0 || n_row_blocks <= 0) return 0;
+    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
+        return (int)hipErrorInvalidValue;
+    if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
+    const int G = Hq / Hkv;
+    if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
+    if (n_splits > 65535) return (int)hipErrorInvalidValue;
+    const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
+    const dim3 grid((unsigned)((tasks + 3) / 4), n_splits);
+#define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
+        token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, Hq, Hkv, BS, scale, \
+        window, split_len, n_splits, group_pad_log2
+    if (row_tiles == 1)
+        hipLaunchKernelGGL(paged_attn_mfma_kernel<1>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
+    else if (row_tiles == 2)
+        hipLaunchKernelGGL(paged_attn_mfma_kernel<2>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
+    else if (row_tiles == 4)
+        hipLaunchKernelGGL(paged_attn_mfma_kernel<4>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
+    else
+        return (int)hipErrorInvalidValue;
+#undef SOC_MFMA_ARGS
+    int err = soc_last_error();
+    if (err || n_splits == 1) return err;
+    hipLaunchKernelGGL(paged_attn_merge_kernel, dim3(Hq, N), dim3(64), 0, stream, part_o, part_ml,
+                       (bf16*)out, Hq, n_splits);
+    return soc_last_error();
+}
+
 SOC_EXPORT int soc_attention_head_dim() { return D; }

@@ -53,6 +53,7 @@ _GEMM_SIGNATURES = {
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P]}
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
+    "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
     "soc_attention_head_dim": [],
 }
 
@@ -80,6 +81,9 @@ class HipKernels:
         _declare(self._gemm, _GEMM_SIGNATURES)
         _declare(self._sampling, _SAMPLING_SIGNATURES)
         self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
+        self.attention_row_tiles = None     # row tiles per wave of the MFMA kernel, override
+        self.attention_mfma = True          # bfloat16 takes the MFMA kernel
+        self._decode_blocks = None
 
     # -- helpers -----------------------------------------------------------------------------
     def _stream(self):
@@ -278,6 +282,43 @@ class HipKernels:
         split_len = ((max_keys + n - 1) // n + 63) // 64 * 64
         return split_len, (max_keys + split_len - 1) // split_len
 
+    def _row_blocks(self, ctx, n_tokens, tokens_per_block):
+        """int32 [blocks, 2] on the device: (first token, tokens) of each run of at most
+        ``tokens_per_block`` tokens of one sequence."""
+        import numpy as np
+        host = getattr(ctx, "host", None)
+        if host is None or "seq_qstart" not in host or tokens_per_block == 1 or ctx.max_q_len == 1:
+            # every token alone (always right; what a decode step is anyway)
+            if self._decode_blocks is None or self._decode_blocks.shape[0] < n_tokens:
+                n = max(n_tokens, 1024)
+                t = torch.stack([torch.arange(n, dtype=torch.int32), torch.ones(n, dtype=torch.int32)], 1)
+                self._decode_blocks = t.contiguous().to(self.device)
+            return self._decode_blocks[:n_tokens], n_tokens
+        cache = host.setdefault("row_blocks", {})
+        if tokens_per_block not in cache:
+            qstart = host["seq_qstart"].astype(np.int64)
+            lens = qstart[1:] - qstart[:-1]
+            counts = (lens + tokens_per_block - 1) // tokens_per_block
+            seq = np.repeat(np.arange(len(lens)), counts)
+            j = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
+            first = qstart[seq] + j * tokens_per_block
+            n = np.minimum(tokens_per_block, lens[seq] - j * tokens_per_block)
+            blocks = np.stack([first, n], 1).astype(np.int32)
+            cache[tokens_per_block] = (torch.from_numpy(blocks).to(self.device), len(blocks))
+        return cache[tokens_per_block]
+
+    def plan_mfma(self, n_blocks, n_kv_heads, group, max_keys):
+        """(split_len, n_splits) for the MFMA kernel: enough waves to fill the GPU, no split
+        shorter than 64 keys. Splits are over absolute key indices."""
+        if self.attention_splits is not None:
+            split_len, n_splits = self.attention_splits
+            split_len = max(16, (min(split_len, 1 << 24) + 15) // 16 * 16)
+            return split_len, max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
+        waves = n_blocks * n_kv_heads * ((group + 15) // 16)
+        n = max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64))
+        split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
+        return split_len, (max_keys + split_len - 1) // split_len
+
     def paged_attention(self, q, slot, ctx, scale, window=None):
         """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""
         N, Hq, D = q.shape
@@ -291,8 +332,29 @@ class HipKernels:
         lib = self._attention_lib(D)
         out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
         w = int(window) if window else 0
+        G = Hq // Hkv
+        if self.dtype == torch.bfloat16 and self.attention_mfma:
+            gpl = max(0, (min(G, 16) - 1).bit_length())
+            decode = getattr(ctx, "max_q_len", 1) == 1
+            rt = self.attention_row_tiles or (1 if decode else 2 if D <= 128 else 1)
+            tokens_per_block = max(1, (16 * rt) >> gpl)
+            blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
+            split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
+            part_o = part_ml = None
+            if n_splits > 1:
+                part_o = torch.empty((N, Hq, n_splits, D), dtype=torch.float32, device=self.device)
+                part_ml = torch.empty((N, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
+            if N > 65535:
+                raise KernelError("more than 65535 tokens in one attention call")
+            _check(lib.soc_paged_attention_mfma(
+                _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+                c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
+                c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), c_int(N), c_int(Hq), c_int(Hkv),
+                c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
+                c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
+            return out
         max_keys = ctx.max_ctx_len if not w else min(w, ctx.max_ctx_len)
-        split_len, n_splits = self.plan_splits(N, Hkv, Hq // Hkv, max_keys)
+        split_len, n_splits = self.plan_splits(N, Hkv, G, max_keys)
         part_o = part_ml = None
         if n_splits > 1:
             part_o = torch.empty((N, Hq, n_splits, D), dtype=torch.float32, device=self.device)

@@ -139,9 +139,16 @@ def make_paged_case(lens, Hq, Hkv, D, bs, dtype, seed, width=None, spare=5):
 
 
 def ctx_for(token_rows, positions):
+    """Device arrays plus the host view of the sequences: a sequence is a run of tokens of
+    one row at consecutive positions."""
+    import numpy as np
+    starts = [0] + [t for t in range(1, len(positions))
+                    if token_rows[t] != token_rows[t - 1] or positions[t] != positions[t - 1] + 1]
+    qstart = np.array(starts + [len(positions)], dtype=np.int32)
     return SimpleNamespace(positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
                            token_rows=torch.tensor(token_rows, dtype=torch.int32, device=DEV),
-                           max_ctx_len=max(positions) + 1)
+                           max_ctx_len=max(positions) + 1, max_q_len=int(np.diff(qstart).max()),
+                           host={"seq_qstart": qstart})
 
 
 def dense_attention(q, dense, token_rows, positions, scale, window=None):
@@ -190,8 +197,11 @@ def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     q = rnd((len(rows), Hq, D), dtype, 9)
     for window in (None, 1, 7, 16, 64):
         want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
-        got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
-        close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+        for row_tiles, splits in ((None, None), (1, (32, 5)), (2, None), (4, (64, 3)), (4, None)):
+            hip.attention_row_tiles, hip.attention_splits = row_tiles, splits
+            got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
+            close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+    hip.attention_row_tiles = hip.attention_splits = None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
