@@ -362,13 +362,18 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     }
 
-    // Global loads of one tile: this lane's K slices and its share of the V tile. Keys that no
-    // row of the block can see are not read at all: zeros stand in for them, so that whatever
-    // lies in stale slots or in the null page (inf, NaN) never meets a product.
-    auto fetch = [&](int key0, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
+    // Page of this lane's key of a tile (lanes 0..15 of every lane group hold keys 0..15).
+    // Keys that no row of the block can see get page -1 and are never read.
+    auto lookup = [&](int key0) -> int {
         const int key = key0 + li;
-        if (key >= kmin && key < khi) {
-            const int page = table[key / BS];
+        return (key >= kmin && key < khi) ? table[key / BS] : -1;
+    };
+    // Global loads of one tile: this lane's K slices and its share of the V tile. Zeros
+    // stand in for keys that are not read, so that whatever lies in stale slots or in the
+    // null page (inf, NaN) never meets a product.
+    auto fetch = [&](int key0, int page, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
+        const int key = key0 + li;
+        if (page >= 0) {
             const bf16* krow = k_pool + ((size_t)page * Hkv * BS + (size_t)kvh * BS + key % BS) * D;
 #pragma unroll
             for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
@@ -379,24 +384,18 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
             const int c = lane + 64 * j;
-            if (V_CHUNKS % 64 == 0 || c < V_CHUNKS) {
-                const int vk = c / (D / 8), part = c % (D / 8);
-                const int vkey = key0 + vk;
-                if (vkey >= kmin && vkey < khi)
-                    vr[j] = *reinterpret_cast<const uint4*>(
-                        v_pool + ((size_t)table[vkey / BS] * Hkv * BS + (size_t)kvh * BS + vkey % BS) * D + part * 8);
-                else
-                    vr[j] = make_uint4(0u, 0u, 0u, 0u);
-            }
+            const int vk = (c / (D / 8)) & 15, part = c % (D / 8);
+            const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
+            if ((V_CHUNKS % 64 == 0 || c < V_CHUNKS) && vpage >= 0)
+                vr[j] = *reinterpret_cast<const uint4*>(
+                    v_pool + ((size_t)vpage * Hkv * BS + (size_t)kvh * BS + (key0 + vk) % BS) * D + part * 8);
+            else
+                vr[j] = make_uint4(0u, 0u, 0u, 0u);
         }
     };
 
-    KFrag kf_cur, kf_next;
-    uint4 vr_cur[V_PER_LANE], vr_next[V_PER_LANE];
-    if (klo < khi) fetch(klo, kf_cur, vr_cur);
-    for (int key0 = klo; key0 < khi; key0 += 16) {
-        const bool more = key0 + 16 < khi;
-        if (more) fetch(key0 + 16, kf_next, vr_next);
+    // One tile: V to LDS, scores, online softmax, weighted values.
+    auto compute = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE]) {
         // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk)
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
@@ -404,12 +403,11 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             if (V_CHUNKS % 64 == 0 || c < V_CHUNKS) {
                 const int vk = c / (D / 8), part = c % (D / 8);
                 uint2* dst = reinterpret_cast<uint2*>(&vl[vk * V_STRIDE + part * 8]);
-                dst[0] = make_uint2(vr_cur[j].x, vr_cur[j].y);
-                dst[1] = make_uint2(vr_cur[j].z, vr_cur[j].w);
+                dst[0] = make_uint2(vr[j].x, vr[j].y);
+                dst[1] = make_uint2(vr[j].z, vr[j].w);
             }
         }
         __builtin_amdgcn_wave_barrier();
-        // scores and softmax per row tile
         s16x4_t pf[RT];
         bool any_rescale = false;
         float alpha[RT];
@@ -417,7 +415,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         for (int rt = 0; rt < RT; ++rt) {
             f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < QK_STEPS; ++kk) s = qk_mfma(kf_cur.v[kk], qf[rt][kk], s);
+            for (int kk = 0; kk < QK_STEPS; ++kk) s = qk_mfma(kf.v[kk], qf[rt][kk], s);
             float sv[4];
             float mx = -INFINITY;
 #pragma unroll
@@ -463,11 +461,29 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vt, pf[rt], o[rt][j], 0, 0, 0);
         }
         __builtin_amdgcn_wave_barrier();
-        if (more) {
-            kf_cur = kf_next;
-#pragma unroll
-            for (int j = 0; j < V_PER_LANE; ++j) vr_cur[j] = vr_next[j];
-        }
+    };
+
+    // Three tiles are in flight per wave (48 keys): HBM latency is several times the time one
+    // tile takes to compute. Buffer b holds tiles b, b + 3, b + 6, ... of the wave's range;
+    // the page of a tile is looked up three steps before its loads are issued.
+    KFrag kf0, kf1, kf2;
+    uint4 vr0[V_PER_LANE], vr1[V_PER_LANE], vr2[V_PER_LANE];
+    int pg0 = -1, pg1 = -1, pg2 = -1;
+    if (klo < khi) fetch(klo, lookup(klo), kf0, vr0);
+    if (klo + 16 < khi) fetch(klo + 16, lookup(klo + 16), kf1, vr1);
+    if (klo + 32 < khi) fetch(klo + 32, lookup(klo + 32), kf2, vr2);
+    if (klo + 48 < khi) pg0 = lookup(klo + 48);
+    if (klo + 64 < khi) pg1 = lookup(klo + 64);
+    if (klo + 80 < khi) pg2 = lookup(klo + 80);
+    for (int key0 = klo; key0 < khi; key0 += 48) {
+        compute(key0, kf0, vr0);
+        if (key0 + 48 < khi) { fetch(key0 + 48, pg0, kf0, vr0); pg0 = lookup(key0 + 96); }
+        if (key0 + 16 >= khi) break;
+        compute(key0 + 16, kf1, vr1);
+        if (key0 + 64 < khi) { fetch(key0 + 64, pg1, kf1, vr1); pg1 = lookup(key0 + 112); }
+        if (key0 + 32 >= khi) break;
+        compute(key0 + 32, kf2, vr2);
+        if (key0 + 80 < khi) { fetch(key0 + 80, pg2, kf2, vr2); pg2 = lookup(key0 + 128); }
     }
 
     // finish: the row sum is spread over the four lanes of the row's column
