@@ -50,8 +50,10 @@ class PagedGroup:
     def __init__(self, need: PagedKV, max_rows, table_width, block_size, num_blocks, dtype, device):
         self.need, self.block_size, self.table_width = need, block_size, table_width
         self.allocator = BlockAllocator(num_blocks)
-        self.host_table = np.zeros((max_rows, table_width), dtype=np.int32)
-        self.table = torch.zeros((max_rows, table_width), dtype=torch.int32, device=device)
+        # one row more than can be opened: the null row, whose entries all point at the null
+        # page, stands in for the padding rows of a fixed-width (captured) decode step
+        self.host_table = np.zeros((max_rows + 1, table_width), dtype=np.int32)
+        self.table = torch.zeros((max_rows + 1, table_width), dtype=torch.int32, device=device)
         # per row: number of logical blocks ever covered, and the first one still held
         self.covered = [0] * max_rows
         self.first_live = [0] * max_rows
@@ -162,7 +164,7 @@ class CacheManager:
                 k, v = group.pools[slot_id]
                 self._slots.append(PagedSlot(k, v, group.table, block_size, need.window))
             elif isinstance(need, RowState):
-                state = torch.zeros((max_rows,) + tuple(need.shape), dtype=torch.float32, device=device)
+                state = torch.zeros((max_rows + 1,) + tuple(need.shape), dtype=torch.float32, device=device)
                 self._slots.append(StateSlot(state))
             elif need is None:
                 self._slots.append(None)
@@ -289,6 +291,11 @@ class CacheManager:
 
     def slot(self, slot_id: int):
         return self._slots[slot_id]
+
+    @property
+    def null_row(self) -> int:
+        """A row that is never opened: all its table entries are the null page."""
+        return self.max_rows
 
     @property
     def n_free_pages(self) -> int:

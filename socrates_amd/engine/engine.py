@@ -113,7 +113,7 @@ class Engine:
             return 0
         entries = [StepEntry(p.request.row, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
                    for p in plan]
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, borrow=True)
         wanted = [p for p in plan if p.wants_logits]
         tokens = self.sampler.sample(logits, [p.request.row for p in wanted])
         for p in plan:

@@ -17,7 +17,7 @@ from ..cache import CacheManager
 from ..config import load_config
 from ..parts import DecoderModel, cache_needs, expected_tensors
 from ..weights import load_weights
-from .batch import StepEntry, build_context
+from .batch import StepContext, StepEntry, build_context
 
 
 class ModelRunner:
@@ -25,6 +25,8 @@ class ModelRunner:
         self.model, self.cache = model, cache
         self.ops = model.ops
         self.vocab_size = model.plan.vocab_size
+        self._graphs = None              # width -> captured decode step, once enable_graphs ran
+        self._graph_max = 0
 
     @classmethod
     def from_folder(cls, folder, dtype, device, max_rows, max_len, block_size, num_blocks, ops=None):
@@ -45,11 +47,16 @@ class ModelRunner:
         return runner
 
     @torch.no_grad()
-    def step(self, entries: List[StepEntry]) -> torch.Tensor:
+    def step(self, entries: List[StepEntry], borrow: bool = False) -> torch.Tensor:
         """Returns float32 logits [wanted places, vocab], in the order of the entries and of
         each entry's ``want``. Raises OutOfBlocks if the pages do not suffice (lengths
-        are then unchanged; pages already taken stay with their rows)."""
+        are then unchanged; pages already taken stay with their rows). ``borrow``: the
+        caller uses the logits before the next step, so a captured step may hand out its own
+        output buffer instead of a copy."""
         cache = self.cache
+        if (self._graphs is not None and len(entries) <= self._graph_max
+                and all(len(e.tokens) == 1 for e in entries)):
+            return self._step_captured(entries, borrow)
         starts = [cache.length(e.row) for e in entries]
         ctx = build_context(entries, starts, self.ops.device, self.vocab_size)
         for e, start in zip(entries, starts):
@@ -59,3 +66,79 @@ class ModelRunner:
         for e in entries:
             cache.advance(e.row, len(e.tokens))
         return logits
+
+    # -- decode steps replayed from HIP graphs -----------------------------------------------------
+    # The reference compiles its decode step with CUDA graphs, one per batch width
+    # (model/inference_paged.py:99-130). Here a step in which every request brings one token
+    # is replayed from a graph captured for its width (rounded up to a bucket; the padding
+    # rows use the cache's null row, so they read and write the null page only). The graph's
+    # inputs live at fixed addresses and are filled by one copy per step; key splits of the
+    # attention kernel are planned for the longest context the cache allows, so the launch
+    # shape never depends on a request's length.
+    _BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+
+    def enable_graphs(self, max_width: int) -> None:
+        if self.ops.device.type != "cuda":
+            return                       # a stand-in kernel set on the CPU has nothing to capture
+        self._graphs = {}
+        self._graph_max = max_width
+
+    def _bucket(self, n: int) -> int:
+        for b in self._BUCKETS:
+            if b >= n:
+                return min(b, max(self._graph_max, n))
+        return n
+
+    def _capture(self, width: int):
+        dev = self.ops.device
+        inputs = torch.zeros((3, width), dtype=torch.int32, device=dev)
+        inputs[2].fill_(self.cache.null_row)
+        staging = torch.zeros((3, width), dtype=torch.int32).pin_memory()
+        arange = torch.arange(width + 1, dtype=torch.int32, device=dev)
+        ctx = StepContext(
+            n_tokens=width, n_seqs=width, n_want=width, token_ids=inputs[0], positions=inputs[1],
+            token_rows=inputs[2], seq_rows=inputs[2], seq_qstart=arange, seq_ctx=inputs[1],
+            want_index=arange[:width], max_q_len=1, max_ctx_len=self.cache.max_len, host={})
+        stream = torch.cuda.Stream(device=dev)
+        stream.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(stream):
+            self.model.forward(ctx, self.cache)          # warm up outside the capture
+        torch.cuda.current_stream(dev).wait_stream(stream)
+        torch.cuda.synchronize(dev)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            logits = self.model.forward(ctx, self.cache)
+        # The graph holds raw addresses: every tensor it reads (the inputs, and ``arange``
+        # through ctx) has to live as long as the graph, so ctx is kept beside it.
+        return graph, inputs, staging, logits, ctx
+
+    def _step_captured(self, entries: List[StepEntry], borrow: bool) -> torch.Tensor:
+        cache = self.cache
+        n = len(entries)
+        rows = [e.row for e in entries]
+        if len(set(rows)) != n:
+            raise ValueError("a cache row appears twice in one step")
+        width = self._bucket(n)
+        if width not in self._graphs:
+            self._graphs[width] = self._capture(width)
+        graph, inputs, staging, logits, _ctx = self._graphs[width]
+        host = staging.numpy()
+        host[0, n:], host[1, n:], host[2, n:] = 0, 0, cache.null_row
+        for i, e in enumerate(entries):
+            token = int(e.tokens[0])
+            if not 0 <= token < self.vocab_size:
+                raise ValueError(f"entry {i}: token id outside [0, {self.vocab_size})")
+            if any(j != 0 for j in e.want):
+                raise ValueError(f"entry {i}: wanted place outside its one token")
+            start = cache.length(e.row)
+            cache.reserve(e.row, start + 1)
+            host[0, i], host[1, i], host[2, i] = token, start, e.row
+        cache.sync()
+        inputs.copy_(staging, non_blocking=True)
+        graph.replay()
+        for e in entries:
+            cache.advance(e.row, 1)
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if len(wanted) == n:
+            return logits[:n] if borrow else logits[:n].clone()
+        return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]

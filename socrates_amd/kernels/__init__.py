@@ -289,8 +289,9 @@ class HipKernels:
         host = getattr(ctx, "host", None)
         if host is None or "seq_qstart" not in host or tokens_per_block == 1 or ctx.max_q_len == 1:
             # every token alone (always right; what a decode step is anyway)
-            if self._decode_blocks is None or self._decode_blocks.shape[0] < n_tokens:
-                n = max(n_tokens, 1024)
+            if self._decode_blocks is None:
+                # allocated once for the largest call: captured graphs keep its address
+                n = 65535
                 t = torch.stack([torch.arange(n, dtype=torch.int32), torch.ones(n, dtype=torch.int32)], 1)
                 self._decode_blocks = t.contiguous().to(self.device)
             return self._decode_blocks[:n_tokens], n_tokens
