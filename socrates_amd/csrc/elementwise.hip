@@ -35,43 +35,55 @@ SOC_EXPORT int soc_embedding(const int* ids, const void* table, float* out, int 
 // ---------------------------------------------------------------------------------------------
 // In place: r = residual[n] + delta[n]; residual[n] = r; out[n] = r / sqrt(mean(r^2) + eps) * w.
 // With `rows`: n = rows[i], nothing is written back, out has one row per index.
+// delta is either one tensor [N, d] of the compute type, or n_partials float32 tensors
+// [n_partials, N, d] (split-K partial sums of a matrix product) that are added in order.
 template <typename T>
 __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __restrict__ delta,
-                                   const float* __restrict__ w, T* __restrict__ out,
-                                   const int* __restrict__ rows, int d, float eps) {
+                                   const float* __restrict__ partials, int n_partials,
+                                   size_t partial_stride, const float* __restrict__ w,
+                                   T* __restrict__ out, const int* __restrict__ rows, int d, float eps) {
     __shared__ float scratch[16];
     const int i = blockIdx.x;
     const int n = rows ? rows[i] : i;
     float* r = residual + (size_t)n * d;
     const T* dl = delta ? delta + (size_t)n * d : nullptr;
+    const float* dp = partials ? partials + (size_t)n * d : nullptr;
     T* o = out + (size_t)i * d;
-    float ss = 0.f;
-    for (int j = threadIdx.x; j < d; j += blockDim.x) {
+    const bool adds = dl || dp;
+    auto summed = [&](int j) {
         float v = r[j];
         if (dl) v += to_float(dl[j]);
-        if (!rows && dl) r[j] = v;
+        if (dp) for (int s = 0; s < n_partials; ++s) v += dp[s * partial_stride + j];
+        return v;
+    };
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < d; j += blockDim.x) {
+        const float v = summed(j);
+        if (!rows && adds) r[j] = v;
         ss += v * v;
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);
     for (int j = threadIdx.x; j < d; j += blockDim.x) {
-        float v = r[j];
-        if (rows && dl) v += to_float(dl[j]);
+        const float v = (rows && adds) ? summed(j) : r[j];
         o[j] = from_float<T>(v * inv * w[j]);
     }
 }
 
-SOC_EXPORT int soc_add_rmsnorm(float* residual, const void* delta, const float* w, void* out,
-                               const int* rows, int n_out, int d, float eps, int dtype,
-                               hipStream_t stream) {
+SOC_EXPORT int soc_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
+                               long long partial_stride, const float* w, void* out, const int* rows,
+                               int n_out, int d, float eps, int dtype, hipStream_t stream) {
     if (n_out <= 0) return 0;
+    if (delta && partials) return (int)hipErrorInvalidValue;
     const int threads = d >= 2048 ? 512 : 256;
     if (dtype == 0)
         hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, stream, residual,
-                           (const float*)delta, w, (float*)out, rows, d, eps);
+                           (const float*)delta, partials, n_partials, (size_t)partial_stride, w,
+                           (float*)out, rows, d, eps);
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, dim3(n_out), dim3(threads), 0, stream, residual,
-                           (const bf16*)delta, w, (bf16*)out, rows, d, eps);
+                           (const bf16*)delta, partials, n_partials, (size_t)partial_stride, w,
+                           (bf16*)out, rows, d, eps);
     return soc_last_error();
 }
 

@@ -191,92 +191,195 @@ SOC_EXPORT int soc_gemm_bf16_mfma(const void* A, const void* W, void* C, int M, 
 }
 
 // ---------------------------------------------------------------------------------------------
-constexpr int SK_UNROLL = 4;            // 16-byte loads of W in flight per lane
-constexpr int SK_MAX_PARTS = 32;        // waves x m-tiles whose partials fit the LDS buffer
+// (A zero operand below is always written as a prvalue: `cond ? *p : zero` with a named
+// `zero` is an lvalue conditional, which selects between a global and a stack address and
+// then loads through a generic pointer.)
+// Skinny GEMM (M <= 64). A workgroup owns RW tiles of 16 rows of W and one of `k_splits`
+// ranges of K; its waves split that range. For every 32 k a lane loads one 16-byte slice of
+// each of its RW weight rows and one slice of X per 16 rows of M: a slice of X is used RW
+// times, which keeps the re-reading of X (it comes from L2 for every workgroup) well below
+// the weight traffic. Two buffers of SK_UNROLL slices keep the loads of the next 128 k in
+// flight while the MFMAs of the current ones run. With k_splits > 1 the workgroups of one
+// row tile write float32 partial sums [k_splits, M, N] that the consumer adds in order (the
+// residual-add + norm kernel does).
+constexpr int SK_UNROLL = 4;            // 16-byte slices per lane, row and buffer (4 x 32 = 128 k)
+constexpr int SK_STEP = 32 * SK_UNROLL;
+constexpr int SK_MAX_WAVES = 8;
 
-template <typename TC, int MT>
-__global__ void __launch_bounds__(1024)
+template <int MT, int RW> struct SkBuf { uint4 w[RW][SK_UNROLL]; uint4 x[MT][SK_UNROLL]; };
+
+template <typename TC, int MT, int RW>
+__global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
-                        int M, int N, int K, int k_per_wave) {
-    __shared__ float red[SK_MAX_PARTS * 256];
+                        float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
+                        int k_per_wave) {
+    __shared__ float red[SK_MAX_WAVES * MT * RW * 256];
     const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * 16 * RW;
     const int li = lane % 16, lk = (lane / 16) * 8;
-    const int k_begin = wave * k_per_wave, k_end = min(K, k_begin + k_per_wave);
-    const bool w_row_ok = n0 + li < N;
-    const bf16* w_row = W + (size_t)(w_row_ok ? n0 + li : 0) * K;
-
-    f32x4 acc[MT];
+    const int split_begin = blockIdx.y * k_per_split;
+    const int split_end = min(K, split_begin + k_per_split);
+    const int k_begin = split_begin + wave * k_per_wave;
+    const int k_end = min(split_end, k_begin + k_per_wave);
+    // Element offsets of this lane's rows (offsets, not pointers: the loads stay global
+    // loads); a row outside the matrix is never loaded.
+    size_t w_off[RW];
+    bool w_ok[RW];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    for (int k0 = k_begin; k0 < k_end; k0 += 32 * SK_UNROLL) {
-        uint4 wf[SK_UNROLL];
-#pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u) {
-            const int k = k0 + 32 * u + lk;
-            wf[u] = (w_row_ok && k < k_end) ? *reinterpret_cast<const uint4*>(w_row + k)
-                                            : make_uint4(0u, 0u, 0u, 0u);
-        }
-#pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u) {
-            const int k = k0 + 32 * u + lk;
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const int m = t * 16 + li;
-                uint4 xf = (m < M && k < k_end) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k)
-                                                : make_uint4(0u, 0u, 0u, 0u);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    *reinterpret_cast<bf16x8*>(&wf[u]), *reinterpret_cast<bf16x8*>(&xf), acc[t], 0, 0, 0);
-            }
-        }
+    for (int r = 0; r < RW; ++r) {
+        w_ok[r] = n0 + r * 16 + li < N;
+        w_off[r] = (size_t)(w_ok[r] ? n0 + r * 16 + li : 0) * K + lk;
     }
-    // acc[t][r] is the partial of C[m = 16 t + lane % 16][n = n0 + 4 * (lane / 16) + r]
+    size_t x_off[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        x_ok[t] = t * 16 + li < M;
+        x_off[t] = (size_t)(x_ok[t] ? t * 16 + li : 0) * K + lk;
+    }
+    f32x4 acc[MT][RW];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[((wave * MT + t) * 64 + lane) * 4 + r] = acc[t][r];
+        for (int r = 0; r < RW; ++r) acc[t][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // Full steps of 128 k load without any predicate (a row outside the matrix reads row 0
+    // and its results are dropped at the store), so the loop body is straight-line code and
+    // the loads of the next step stay in flight under the MFMAs of the current one.
+#define SK_LOAD(B, K0)                                                                              \
+    _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u) {                                          \
+        _Pragma("unroll") for (int r = 0; r < RW; ++r)                                               \
+            B.w[r][u] = *reinterpret_cast<const uint4*>(W + w_off[r] + (K0) + 32 * u);               \
+        _Pragma("unroll") for (int t = 0; t < MT; ++t)                                               \
+            B.x[t][u] = *reinterpret_cast<const uint4*>(X + x_off[t] + (K0) + 32 * u);               \
+    }
+#define SK_COMPUTE(B)                                                                               \
+    _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u)                                            \
+        _Pragma("unroll") for (int t = 0; t < MT; ++t)                                               \
+            _Pragma("unroll") for (int r = 0; r < RW; ++r)                                           \
+                acc[t][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                 \
+                    __builtin_bit_cast(bf16x8, B.w[r][u]), __builtin_bit_cast(bf16x8, B.x[t][u]),    \
+                    acc[t][r], 0, 0, 0);
+
+    SkBuf<MT, RW> b0, b1;
+    const int steps = max(k_end - k_begin, 0) / SK_STEP;
+    const int k_full = k_begin + steps * SK_STEP;
+    if (steps > 0) {
+        SK_LOAD(b0, k_begin)
+        int s = 1;
+        // steady state: no branch between a load and the MFMAs that must not wait for it
+        for (; s + 1 < steps; s += 2) {
+            SK_LOAD(b1, k_begin + s * SK_STEP)
+            SK_COMPUTE(b0)
+            SK_LOAD(b0, k_begin + (s + 1) * SK_STEP)
+            SK_COMPUTE(b1)
+        }
+        if (s < steps) {
+            SK_LOAD(b1, k_begin + s * SK_STEP)
+            SK_COMPUTE(b0)
+            SK_COMPUTE(b1)
+        } else {
+            SK_COMPUTE(b0)
+        }
+    }
+#undef SK_LOAD
+    // The last, partial step of the range (only where K is no multiple of 128): slices past
+    // the end contribute zeros.
+    if (k_full < k_end) {
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; ++u) {
+            const int kk = k_full + 32 * u;
+            const bool in = kk + lk < k_end;
+#pragma unroll
+            for (int r = 0; r < RW; ++r)
+                b0.w[r][u] = in ? *reinterpret_cast<const uint4*>(W + w_off[r] + kk) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                b0.x[t][u] = in ? *reinterpret_cast<const uint4*>(X + x_off[t] + kk) : make_uint4(0u, 0u, 0u, 0u);
+        }
+        SK_COMPUTE(b0)
+    }
+#undef SK_COMPUTE
+    // acc[t][r][e] is the partial of C[m = 16 t + lane % 16][n = n0 + 16 r + 4 * (lane / 16) + e]
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < RW; ++r)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                red[(((wave * MT + t) * RW + r) * 64 + lane) * 4 + e] = acc[t][r][e];
     __syncthreads();
-    for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
-        const int t = idx / 256, ln = (idx % 256) / 4, r = idx % 4;
+    for (int idx = tid; idx < MT * RW * 256; idx += blockDim.x) {
+        const int tr = idx / 256, ln = (idx % 256) / 4, e = idx % 4;
+        const int t = tr / RW, r = tr % RW;
         float sum = 0.f;
-        for (int w = 0; w < n_waves; ++w) sum += red[((w * MT + t) * 64 + ln) * 4 + r];
-        const int m = t * 16 + ln % 16, n = n0 + 4 * (ln / 16) + r;
-        if (m < M && n < N) C[(size_t)m * N + n] = from_float<TC>(sum);
+        for (int w = 0; w < n_waves; ++w) sum += red[((w * MT * RW + tr) * 64 + ln) * 4 + e];
+        const int m = t * 16 + ln % 16, n = n0 + r * 16 + 4 * (ln / 16) + e;
+        if (m < M && n < N) {
+            if (Cpart) Cpart[((size_t)blockIdx.y * M + m) * N + n] = sum;
+            else C[(size_t)m * N + n] = from_float<TC>(sum);
+        }
     }
 }
 
-template <typename TC, int MT>
-static int launch_skinny(const void* X, const void* W, void* C, int M, int N, int K, int n_waves,
-                         hipStream_t stream) {
-    int k_per_wave = ((K + n_waves - 1) / n_waves + 31) / 32 * 32;
-    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT>), dim3((N + 15) / 16), dim3(n_waves * 64), 0,
-                       stream, (const bf16*)X, (const bf16*)W, (TC*)C, M, N, K, k_per_wave);
+template <typename TC, int MT, int RW>
+static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N, int K,
+                         int n_waves, int k_splits, hipStream_t stream) {
+    // ranges are multiples of the 128-k step, so only the end of K can be a partial step
+    const int k_per_split = ((K + k_splits - 1) / k_splits + SK_STEP - 1) / SK_STEP * SK_STEP;
+    const int k_per_wave = ((k_per_split + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT, RW>), dim3((N + 16 * RW - 1) / (16 * RW), k_splits),
+                       dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (TC*)C, Cpart, M, N,
+                       K, k_per_split, k_per_wave);
     return soc_last_error();
 }
 
-// M <= 64, K a multiple of 8. n_waves (1..16) is how many waves of a workgroup split K;
-// 0 lets the kernel choose from the shape.
-SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, int M, int N, int K,
-                                    int c_dtype, int n_waves, hipStream_t stream) {
+// Shape heuristics shared with the host wrapper (which sizes the partial buffer): rows per
+// workgroup (in tiles of 16), waves of a workgroup, and workgroups that split K, for an
+// [M <= 64] x [N, K] product.
+SOC_EXPORT void soc_gemm_skinny_plan(int M, int N, int K, int allow_split, int* row_tiles, int* n_waves,
+                                     int* k_splits) {
+    // From measurements at K = 2560..9728 on an MI355X: wide outputs have enough row tiles
+    // to fill the GPU with one tile per workgroup; narrow ones need two workgroups per K.
+    int rw, nw, ks = 1;
+    if (M > 16) { rw = 2; nw = N >= 16384 ? 4 : 8; }
+    else if (N >= 16384) { rw = 1; nw = 8; }
+    else if (N >= 4096) { rw = 2; nw = 4; }
+    else if (allow_split && K >= 2048) { rw = 2; nw = 8; ks = 2; }
+    else { rw = 1; nw = 8; }
+    while (nw > 1 && K / (nw * ks) < 128) nw /= 2;
+    while (ks > 1 && K / (nw * ks) < 128) ks /= 2;
+    *row_tiles = rw;
+    *n_waves = nw;
+    *k_splits = ks;
+}
+
+// M <= 64, K a multiple of 8. k_splits == 1: C [M, N] in c_dtype. k_splits > 1: float32
+// partial sums Cpart [k_splits, M, N] (C is not written).
+SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N,
+                                    int K, int c_dtype, int row_tiles, int n_waves, int k_splits,
+                                    hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 8 || K < 8) return (int)hipErrorInvalidValue;
+    if (n_waves < 1 || n_waves > SK_MAX_WAVES || k_splits < 1 || k_splits > 65535)
+        return (int)hipErrorInvalidValue;
+    if ((k_splits > 1) != (Cpart != nullptr)) return (int)hipErrorInvalidValue;
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    if (n_waves <= 0) {
-        const int tiles = (N + 15) / 16;
-        n_waves = tiles >= 2048 ? 4 : (tiles >= 512 ? 8 : 16);
-    }
-    while (n_waves > 1 && (n_waves * MT > SK_MAX_PARTS || K / n_waves < 128)) n_waves /= 2;
-    if (n_waves > 16) n_waves = 16;
-#define SOC_SK(TC_, MT_) return launch_skinny<TC_, MT_>(X, W, C, M, N, K, n_waves, stream)
+    if (row_tiles != 2 && !((row_tiles == 4 || row_tiles == 1) && MT == 1)) return (int)hipErrorInvalidValue;
+#define SOC_SK(TC_, MT_, RW_) \
+    return launch_skinny<TC_, MT_, RW_>(X, W, C, Cpart, M, N, K, n_waves, k_splits, stream)
     if (c_dtype == 0) {
-        if (MT == 1) SOC_SK(float, 1);
-        if (MT == 2) SOC_SK(float, 2);
-        SOC_SK(float, 4);
+        if (MT == 1 && row_tiles == 4) SOC_SK(float, 1, 4);
+        if (MT == 1 && row_tiles == 1) SOC_SK(float, 1, 1);
+        if (MT == 1) SOC_SK(float, 1, 2);
+        if (MT == 2) SOC_SK(float, 2, 2);
+        SOC_SK(float, 4, 2);
     }
-    if (MT == 1) SOC_SK(bf16, 1);
-    if (MT == 2) SOC_SK(bf16, 2);
-    SOC_SK(bf16, 4);
+    if (MT == 1 && row_tiles == 4) SOC_SK(bf16, 1, 4);
+    if (MT == 1 && row_tiles == 1) SOC_SK(bf16, 1, 1);
+    if (MT == 1) SOC_SK(bf16, 1, 2);
+    if (MT == 2) SOC_SK(bf16, 2, 2);
+    SOC_SK(bf16, 4, 2);
 #undef SOC_SK
 }

@@ -11,7 +11,7 @@ is launched, so that a wrong operand is an exception and not a memory fault.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_void_p
+from ctypes import c_float, c_int, c_longlong, c_void_p
 
 import torch
 
@@ -38,7 +38,7 @@ def _check(err, what):
 P, I, F = c_void_p, c_int, c_float
 _EW_SIGNATURES = {
     "soc_embedding": [P, P, P, I, I, I, I, P],
-    "soc_add_rmsnorm": [P, P, P, P, P, I, I, F, I, P],
+    "soc_add_rmsnorm": [P, P, P, I, c_longlong, P, P, P, I, I, F, I, P],
     "soc_rmsnorm": [P, P, P, I, I, F, I, P],
     "soc_swiglu": [P, P, I, I, I, P],
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
@@ -48,7 +48,8 @@ _EW_SIGNATURES = {
 _GEMM_SIGNATURES = {
     "soc_gemm_generic": [P, P, P, I, I, I, I, I, I, P],
     "soc_gemm_bf16_mfma": [P, P, P, I, I, I, I, P],
-    "soc_gemm_bf16_skinny": [P, P, P, I, I, I, I, I, P],
+    "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
+    "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -61,7 +62,7 @@ _ATTENTION_SIGNATURES = {
 def _declare(lib, signatures):
     for name, argtypes in signatures.items():
         fn = getattr(lib, name)
-        fn.argtypes, fn.restype = argtypes, c_int
+        fn.argtypes, fn.restype = argtypes, (None if name.endswith("_plan") else c_int)
 
 
 class HipKernels:
@@ -129,16 +130,23 @@ class HipKernels:
         return out
 
     def add_rmsnorm(self, residual, delta, weight, eps, rows=None):
+        """``delta``: None, a [N, d] tensor of the compute dtype, or float32 partial sums
+        [S, N, d] (what ``linear(..., allow_partial=True)`` returns) that are added in order."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
         self._want(weight, "norm weight", torch.float32, (d,))
-        if delta is not None:
-            self._want(delta, "delta", self.dtype, (N, d))
+        whole = partials = None
+        n_partials = 0
+        if delta is not None and delta.dim() == 3:
+            partials, n_partials = self._want(delta, "partial sums", torch.float32, (delta.shape[0], N, d)), delta.shape[0]
+        elif delta is not None:
+            whole = self._want(delta, "delta", self.dtype, (N, d))
         if rows is not None:
             self._want(rows, "rows", torch.int32)
         n_out = N if rows is None else rows.numel()
         out = torch.empty((n_out, d), dtype=self.dtype, device=self.device)
-        _check(self._ew.soc_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
+        _check(self._ew.soc_add_rmsnorm(_ptr(residual), _ptr(whole), _ptr(partials), c_int(n_partials),
+                                        c_longlong(N * d), _ptr(weight), _ptr(out), _ptr(rows),
                                         c_int(n_out), c_int(d), c_float(eps), c_int(self.code),
                                         self._stream()), "add_rmsnorm")
         return out
@@ -163,9 +171,11 @@ class HipKernels:
         return out
 
     # -- matrix products ------------------------------------------------------------------------
-    def linear(self, x, w, out_dtype=None, n_waves=0):
+    def linear(self, x, w, out_dtype=None, allow_partial=False, row_tiles=0, n_waves=0, k_splits=0):
         """x [M, K] times w [N, K] transposed. float32 operands (either) take the plain
-        float32 kernel; bfloat16 pairs take the MFMA kernels."""
+        float32 kernel; bfloat16 pairs take the MFMA kernels. ``allow_partial``: the consumer
+        (the residual-add + norm kernel) accepts float32 split-K partial sums [S, M, N]; the
+        skinny kernel then spreads a narrow output over more workgroups."""
         self._want(x, "x")
         self._want(w, "weight")
         if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -174,17 +184,31 @@ class HipKernels:
         out_dtype = out_dtype or self.dtype
         if x.dtype not in _DTYPE_CODE or w.dtype not in _DTYPE_CODE or out_dtype not in _DTYPE_CODE:
             raise KernelError(f"linear: dtypes {x.dtype}, {w.dtype}, {out_dtype} are not supported")
-        out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         if M == 0:
-            return out
-        args = (_ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K))
+            return torch.empty((M, N), dtype=out_dtype, device=self.device)
         both_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-        if both_bf16 and K % 8 == 0 and K >= 8:
-            if M <= 64:
-                err = self._gemm.soc_gemm_bf16_skinny(*args, c_int(_DTYPE_CODE[out_dtype]), c_int(n_waves),
-                                                      self._stream())
+        if both_bf16 and K % 8 == 0 and K >= 8 and M <= 64:
+            if not (row_tiles and n_waves and k_splits):
+                rw, nw, ks = c_int(0), c_int(0), c_int(0)
+                self._gemm.soc_gemm_skinny_plan(c_int(M), c_int(N), c_int(K), c_int(1 if allow_partial else 0),
+                                                ctypes.byref(rw), ctypes.byref(nw), ctypes.byref(ks))
+                row_tiles, n_waves = row_tiles or rw.value, n_waves or nw.value
+                k_splits = k_splits or ks.value
+            if k_splits > 1:
+                part = torch.empty((k_splits, M, N), dtype=torch.float32, device=self.device)
+                out, c_ptr, p_ptr = part, None, _ptr(part)
             else:
-                err = self._gemm.soc_gemm_bf16_mfma(*args, c_int(_DTYPE_CODE[out_dtype]), self._stream())
+                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+                c_ptr, p_ptr = _ptr(out), None
+            _check(self._gemm.soc_gemm_bf16_skinny(_ptr(x), _ptr(w), c_ptr, p_ptr, c_int(M), c_int(N), c_int(K),
+                                                   c_int(_DTYPE_CODE[out_dtype]), c_int(row_tiles),
+                                                   c_int(n_waves), c_int(k_splits), self._stream()),
+                   f"linear [{M}x{K}] x [{N}x{K}]^T")
+            return out
+        out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+        args = (_ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K))
+        if both_bf16 and K % 8 == 0 and K >= 8:
+            err = self._gemm.soc_gemm_bf16_mfma(*args, c_int(_DTYPE_CODE[out_dtype]), self._stream())
         else:
             err = self._gemm.soc_gemm_generic(*args, c_int(_DTYPE_CODE[x.dtype]), c_int(_DTYPE_CODE[w.dtype]),
                                               c_int(_DTYPE_CODE[out_dtype]), self._stream())

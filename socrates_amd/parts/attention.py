@@ -71,7 +71,8 @@ class PagedAttention:
             if write:
                 ops.kv_write(k, v, ctx.positions, ctx.token_rows, slot)
         o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
-        return ops.linear(o, self.w_o)
+        # the block's next norm adds this output to the residual: partial sums are welcome
+        return ops.linear(o, self.w_o, allow_partial=True)
 
 
 register_part(AttentionSpec, PagedAttention)

@@ -25,7 +25,8 @@ class SwiGLU:
 
     def forward(self, x, ctx=None):
         gate_up = self.ops.linear(x, self.w_gate_up)
-        return self.ops.linear(self.ops.swiglu(gate_up), self.w_down)
+        # the block's next norm adds this output to the residual: partial sums are welcome
+        return self.ops.linear(self.ops.swiglu(gate_up), self.w_down, allow_partial=True)
 
 
 register_part(SwiGLUSpec, SwiGLU)

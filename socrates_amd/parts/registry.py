@@ -10,10 +10,11 @@ Interfaces (duck-typed):
 
   every part   ``tensors(spec) -> {local_name: TensorDecl}`` (staticmethod)
                ``__init__(spec, tensors, ops)``
-  norm         ``add_norm(residual, delta, rows=None) -> normed``: adds ``delta`` (or
-               nothing) into the fp32 ``residual`` in place and returns the normed
-               activations in the compute dtype; with ``rows`` it works on those
-               rows only and leaves ``residual`` alone
+  norm         ``add_norm(residual, delta, rows=None) -> normed``: adds ``delta`` (nothing,
+               a [N, d] tensor, or float32 partial sums [S, N, d]) into the fp32
+               ``residual`` in place and returns the normed activations in the compute
+               dtype; with ``rows`` it works on those rows only and leaves ``residual``
+               alone
   position     ``rotary() -> (inv_freq, rotary_dim) | None`` for the fused kernel, and
                ``apply(q, k, positions)`` in place on [N, H, D] tensors
   mixer        ``cache_need(spec) -> PagedKV | RowState | None`` (staticmethod)

@@ -103,6 +103,29 @@ def test_linear(kernel_sets, a_dt, w_dt, c_dt, M, N, K):
         torch.testing.assert_close(got.double(), want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (8, 2560, 9728), (40, 100, 2048), (64, 6144, 2560)])
+def test_linear_split_k_partials(kernel_sets, M, N, K):
+    """Narrow outputs spread K over several workgroups and return float32 partial sums that
+    the residual-add + norm kernel adds in order."""
+    hip, ref = kernel_sets[torch.bfloat16]
+    x, w = rnd((M, K), torch.bfloat16, 6), rnd((N, K), torch.bfloat16, 7, K ** -0.5)
+    want = x.double() @ w.double().T
+    for ks in (0, 1, 2, 4, 7):
+        got = hip.linear(x, w, allow_partial=True, k_splits=ks)
+        if ks > 1:
+            assert got.shape == (ks, M, N) and got.dtype == torch.float32
+        total = got.double().sum(0) if got.dim() == 3 else got.double()
+        torch.testing.assert_close(total, want, atol=2e-2, rtol=2e-2)
+        if got.dim() == 3:
+            res = rnd((M, N), torch.float32, 8)
+            gain = (1 + 0.1 * torch.randn(N)).to(DEV)
+            r1, r2 = res.clone(), res.clone()
+            a = hip.add_rmsnorm(r1, got, gain, 1e-6)
+            b = ref.add_rmsnorm(r2, got, gain, 1e-6)
+            close(a, b, torch.bfloat16)
+            torch.testing.assert_close(r1, r2, atol=1e-5, rtol=1e-5)
+
+
 def test_linear_float32_is_not_reduced_precision(kernel_sets):
     """Values that bfloat16 or a 19-bit matrix mode would round away survive."""
     hip, _ = kernel_sets[torch.float32]

@@ -24,6 +24,11 @@ KINDS = [pytest.param("torch", torch.float32, id="cpu-fp32"),
 TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
 
 
+def whole(t):
+    """A part's output as one tensor: split-K partial sums [S, N, d] are added up."""
+    return t.float().sum(0) if t.dim() == 3 else t.float()
+
+
 def kernels(kind, dtype):
     if kind == "torch":
         from torch_kernels import TorchKernels
@@ -95,7 +100,7 @@ def test_each_part_alone(folders, kind, dtype):
     ffn = build_part(spec.ffn, {n: dev(w[p + "mlp." + n]) for n in ("gate_proj.weight", "up_proj.weight",
                                                                      "down_proj.weight")}, ops)
     xin = dev(x)
-    torch.testing.assert_close(ffn.forward(xin).float().cpu(), plain.swiglu_mlp(xin.float().cpu(), w, p + "mlp."), **tol)
+    torch.testing.assert_close(whole(ffn.forward(xin)).cpu(), plain.swiglu_mlp(xin.float().cpu(), w, p + "mlp."), **tol)
 
     att_tensors = {n: dev(w[p + "self_attn." + n], torch.float32 if "norm" in n else dtype)
                    for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight",
@@ -108,7 +113,7 @@ def test_each_part_alone(folders, kind, dtype):
     ctx = ctx_of(ops, [T])
     got = mixer.forward(xin, ctx, cache.slot(0), True)
     want = plain.attention_layer(xin.float().cpu(), w, p + "self_attn.", cfg, torch.arange(T))
-    torch.testing.assert_close(got.float().cpu(), want, **tol)
+    torch.testing.assert_close(whole(got).cpu(), want, **tol)
 
     block_w = {n: dev(t, torch.float32 if t.dim() == 1 else dtype) for n, t in w.items() if n.startswith(p)}
     block = build_block(spec, block_w, ops)
@@ -117,7 +122,7 @@ def test_each_part_alone(folders, kind, dtype):
     cache.sync()
     residual = dev(x, torch.float32)
     pending = block.forward(residual, None, ctx, cache.slot(0), True)
-    torch.testing.assert_close(residual.cpu() + pending.float().cpu(), plain.block(x, w, 1, cfg, torch.arange(T)), **tol)
+    torch.testing.assert_close(residual.cpu() + whole(pending).cpu(), plain.block(x, w, 1, cfg, torch.arange(T)), **tol)
 
 
 @pytest.mark.parametrize("kind,dtype", KINDS)
@@ -150,7 +155,7 @@ def test_attention_part_with_a_window_in_portions(kind, dtype):
         cache.reserve(row, t + n)
         cache.sync()
         ctx = ctx_of(ops, [n], [t], [row])
-        outs.append(mixer.forward(dev(x[t:t + n]), ctx, cache.slot(0), True).float().cpu())
+        outs.append(whole(mixer.forward(dev(x[t:t + n]), ctx, cache.slot(0), True)).cpu())
         cache.advance(row, n)
         cache.check()
         t += n

@@ -41,6 +41,8 @@ class TorchKernels:
         return x / torch.sqrt(var + eps) * weight.to(self.acc)
 
     def add_rmsnorm(self, residual, delta, weight, eps, rows=None):
+        if delta is not None and delta.dim() == 3:            # split-K partial sums
+            delta = delta.sum(0)
         if rows is not None:
             r = residual[rows.long()].to(self.acc)
             if delta is not None:
@@ -58,7 +60,7 @@ class TorchKernels:
         g, u = gate_up[..., :ff].to(self.acc), gate_up[..., ff:].to(self.acc)
         return (u * (g * torch.sigmoid(g))).to(self.dtype)
 
-    def linear(self, x, w, out_dtype=None):
+    def linear(self, x, w, out_dtype=None, allow_partial=False):
         y = x.to(self.acc) @ w.to(self.acc).T
         return y.to(out_dtype or self.dtype)
 
