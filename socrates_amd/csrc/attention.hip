@@ -514,25 +514,37 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     }
 }
 
-// Merge all n_splits partials of a (token, head); an empty split has m = -inf.
-__global__ void paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                        bf16* __restrict__ out, int Hq, int n_splits) {
-    const int h = blockIdx.x, n = blockIdx.y;
+// Merge all n_splits partials of a (token, head); an empty split has m = -inf. One wave per
+// (token, head): first the splits lie across the lanes (maximum, weights, sum), then the head
+// dimension does, each lane adding its elements over the splits in order.
+__global__ void __launch_bounds__(64)
+paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                        bf16* __restrict__ out, int Hq, int n_splits) {
+    __shared__ float weight[256];
+    const int h = blockIdx.x, n = blockIdx.y, lane = threadIdx.x;
     const size_t base = ((size_t)n * Hq + h) * n_splits;
     float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+    for (int s = lane; s < n_splits; s += SOC_WAVE) M = fmaxf(M, part_ml[(base + s) * 2]);
+    M = wave_max(M);
     float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float ms = part_ml[(base + s) * 2];
-        if (ms != -INFINITY) L += part_ml[(base + s) * 2 + 1] * __expf(ms - M);
-    }
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
-    for (int e = threadIdx.x; e < D; e += blockDim.x) {
-        float A = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
+    for (int s0 = 0; s0 < n_splits; s0 += 256) {           // weights of up to 256 splits at a time
+        float lsum = 0.f;
+        for (int s = s0 + lane; s < min(n_splits, s0 + 256); s += SOC_WAVE) {
             const float ms = part_ml[(base + s) * 2];
-            if (ms != -INFINITY) A += part_o[(base + s) * D + e] * __expf(ms - M);
+            const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+            weight[s - s0] = w;
+            lsum += w * part_ml[(base + s) * 2 + 1];
         }
+        L += wave_sum(lsum);
+        if (s0 + 256 < n_splits) break;                     // (more than 256 splits: handled below)
+    }
+    __syncthreads();
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    const int first = min(n_splits, 256);
+    for (int e = lane; e < D; e += SOC_WAVE) {
+        float A = 0.f;
+#pragma unroll 4
+        for (int s = 0; s < first; ++s) A += part_o[(base + s) * D + e] * weight[s];
         out[((size_t)n * Hq + h) * D + e] = from_float<bf16>(A * inv);
     }
 }
@@ -554,7 +566,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
-    if (n_splits > 65535) return (int)hipErrorInvalidValue;
+    if (n_splits > 256) return (int)hipErrorInvalidValue;        // the merge holds 256 weights
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     const dim3 grid((unsigned)((tasks + 3) / 4), n_splits);
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \

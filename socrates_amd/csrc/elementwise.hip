@@ -150,11 +150,13 @@ SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int dty
 // (q and k only, if gains are given), rotate-half rotation at the token's position (q and k
 // only, if inv_freq is given), then store: q to q_out; k and v into the cache pages of the
 // token's row at its position, or to k_out / v_out when no pools are given.
-// One wave per head; a workgroup of 4 waves walks the heads of one token.
+// One wave per head: workgroup (token, group of 4 heads), no loop, so a decode step's few
+// tokens still spread over many workgroups and the kernel is one short pass.
 #define SOC_MAX_HEAD 256
 
 template <typename T>
-__global__ void qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
+__global__ void __launch_bounds__(256)
+qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                     T* __restrict__ k_out, T* __restrict__ v_out,
                                     T* __restrict__ k_pool, T* __restrict__ v_pool,
                                     const int* __restrict__ block_table, int table_width,
@@ -167,74 +169,65 @@ __global__ void qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q
     const int n = blockIdx.x;
     const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
     const int heads = Hq + 2 * Hkv;
-    const T* row = qkv + (size_t)n * heads * D;
-    const int pos = positions[n];
-    size_t page_base = 0;
-    if (k_pool) {
-        const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
-        page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;     // + kv_head * BS * D
-    }
+    const int h = blockIdx.y * 4 + wave;
+    const bool active = h < heads;
+    const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
+    const T* x = qkv + ((size_t)n * heads + (active ? h : 0)) * D;
+    const int pos = positions ? positions[n] : 0;
     const int half = rotary_dim / 2;
-    // The trip count is the same for all four waves so that the barriers below are uniform.
-    for (int h0 = 0; h0 < heads; h0 += 4) {
-        const int h = h0 + wave;
-        const bool active = h < heads;
-        const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
-        const T* x = row + (size_t)(active ? h : 0) * D;
-        float v[SOC_MAX_HEAD / SOC_WAVE];
-        float ss = 0.f;
+    float v[SOC_MAX_HEAD / SOC_WAVE];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+        const int e = lane + i * SOC_WAVE;
+        v[i] = e < D ? to_float(x[e]) : 0.f;
+        ss += v[i] * v[i];
+    }
+    const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+    if (gain && active) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
         for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
             const int e = lane + i * SOC_WAVE;
-            v[i] = e < D ? to_float(x[e]) : 0.f;
-            ss += v[i] * v[i];
+            if (e < D) v[i] = v[i] * inv * gain[e];
         }
-        const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
-        if (gain && active) {
-            ss = wave_sum(ss);
-            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    if (inv_freq) {                                   // uniform over the workgroup
 #pragma unroll
-            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-                const int e = lane + i * SOC_WAVE;
-                if (e < D) v[i] = v[i] * inv * gain[e];
-            }
+        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+            const int e = lane + i * SOC_WAVE;
+            if (e < D) stage[wave][e] = v[i];
         }
-        if (inv_freq) {
-            const bool rotate = active && (is_q || is_k);
-#pragma unroll
-            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-                const int e = lane + i * SOC_WAVE;
-                if (e < D) stage[wave][e] = v[i];
-            }
-            __syncthreads();
-            if (rotate) {
+        __syncthreads();
+        if (active && (is_q || is_k)) {
 #pragma unroll
             for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
                 const int e = lane + i * SOC_WAVE;
                 if (e < rotary_dim) {
                     const int j = e < half ? e : e - half;
                     const float partner = stage[wave][e < half ? e + half : e - half];
-                    float s, c;
-                    sincosf((float)pos * inv_freq[j], &s, &c);
-                    v[i] = e < half ? v[i] * c - partner * s : v[i] * c + partner * s;
+                    float sn, cs;
+                    sincosf((float)pos * inv_freq[j], &sn, &cs);
+                    v[i] = e < half ? v[i] * cs - partner * sn : v[i] * cs + partner * sn;
                 }
             }
-            }
-            __syncthreads();
         }
-        if (!active) continue;
-        T* dst;
-        if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
-        else {
-            const int kvh = is_k ? h - Hq : h - Hq - Hkv;
-            if (k_pool) dst = (is_k ? k_pool : v_pool) + page_base + (size_t)kvh * BS * D;
-            else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
-        }
+    }
+    if (!active) return;
+    T* dst;
+    if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
+    else {
+        const int kvh = is_k ? h - Hq : h - Hq - Hkv;
+        if (k_pool) {
+            const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
+            dst = (is_k ? k_pool : v_pool) + (((size_t)page * Hkv + kvh) * BS + (size_t)(pos % BS)) * D;
+        } else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
+    }
 #pragma unroll
-        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-            const int e = lane + i * SOC_WAVE;
-            if (e < D) dst[e] = from_float<T>(v[i]);
-        }
+    for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
+        const int e = lane + i * SOC_WAVE;
+        if (e < D) dst[e] = from_float<T>(v[i]);
     }
 }
 
@@ -246,13 +239,16 @@ SOC_EXPORT int soc_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void*
                                 hipStream_t stream) {
     if (N <= 0) return 0;
     if (D > SOC_MAX_HEAD || D < 1) return (int)hipErrorInvalidValue;
+    const int head_groups = (Hq + 2 * Hkv + 3) / 4;
+    if (head_groups > 65535) return (int)hipErrorInvalidValue;
+    const dim3 grid(N, head_groups);
     if (dtype == 0)
-        hipLaunchKernelGGL(qk_norm_rope_kernel<float>, dim3(N), dim3(256), 0, stream, (const float*)qkv,
+        hipLaunchKernelGGL(qk_norm_rope_kernel<float>, grid, dim3(256), 0, stream, (const float*)qkv,
                            (float*)q_out, (float*)k_out, (float*)v_out, (float*)k_pool, (float*)v_pool,
                            block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
                            Hq, Hkv, D, rotary_dim, BS, eps);
     else
-        hipLaunchKernelGGL(qk_norm_rope_kernel<bf16>, dim3(N), dim3(256), 0, stream, (const bf16*)qkv,
+        hipLaunchKernelGGL(qk_norm_rope_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)qkv,
                            (bf16*)q_out, (bf16*)k_out, (bf16*)v_out, (bf16*)k_pool, (bf16*)v_pool,
                            block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
                            Hq, Hkv, D, rotary_dim, BS, eps);

@@ -95,6 +95,57 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
     if (threadIdx.x == 0) out[row] = chosen;
 }
 
+// Greedy choice for many rows at once: a row is cut into chunks, one workgroup per chunk
+// finds its best (value, index), and the last step picks among the chunks, lowest index first.
+constexpr int ARGMAX_THREADS = 256;
+
+__global__ void __launch_bounds__(ARGMAX_THREADS)
+argmax_chunks_kernel(const float* __restrict__ logits, MaxIdx* __restrict__ partial, int V, int chunk) {
+    __shared__ MaxIdx scratch[ARGMAX_THREADS / SOC_WAVE];
+    const int row = blockIdx.y, c = blockIdx.x;
+    const int begin = c * chunk, end = min(V, begin + chunk);
+    const float* x = logits + (size_t)row * V;
+    MaxIdx best = {-INFINITY, 0x7fffffff};
+    for (int i = begin + threadIdx.x; i < end; i += ARGMAX_THREADS) best = better(best, MaxIdx{x[i], i});
+#pragma unroll
+    for (int m = SOC_WAVE / 2; m > 0; m >>= 1) {
+        MaxIdx o = {__shfl_xor(best.v, m, SOC_WAVE), __shfl_xor(best.i, m, SOC_WAVE)};
+        best = better(best, o);
+    }
+    if (threadIdx.x % SOC_WAVE == 0) scratch[threadIdx.x / SOC_WAVE] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        MaxIdx r = scratch[0];
+        for (int w = 1; w < ARGMAX_THREADS / SOC_WAVE; ++w) r = better(r, scratch[w]);
+        partial[(size_t)row * gridDim.x + c] = r;
+    }
+}
+
+__global__ void argmax_pick_kernel(const MaxIdx* __restrict__ partial, int* __restrict__ out, int n_chunks) {
+    const int row = blockIdx.x;
+    MaxIdx best = {-INFINITY, 0x7fffffff};
+    for (int c = threadIdx.x; c < n_chunks; c += SOC_WAVE) best = better(best, partial[(size_t)row * n_chunks + c]);
+#pragma unroll
+    for (int m = SOC_WAVE / 2; m > 0; m >>= 1) {
+        MaxIdx o = {__shfl_xor(best.v, m, SOC_WAVE), __shfl_xor(best.i, m, SOC_WAVE)};
+        best = better(best, o);
+    }
+    if (threadIdx.x == 0) out[row] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
+// logits [n, V] float32 -> out [n] int32. partial: scratch of n * n_chunks (float, int) pairs.
+SOC_EXPORT int soc_argmax(const float* logits, void* partial, int* out, int n, int V, int n_chunks,
+                          hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (V < 1 || n_chunks < 1 || n > 65535) return (int)hipErrorInvalidValue;
+    const int chunk = (V + n_chunks - 1) / n_chunks;
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(n_chunks, n), dim3(ARGMAX_THREADS), 0, stream, logits,
+                       (MaxIdx*)partial, V, chunk);
+    hipLaunchKernelGGL(argmax_pick_kernel, dim3(n), dim3(SOC_WAVE), 0, stream, (const MaxIdx*)partial, out,
+                       n_chunks);
+    return soc_last_error();
+}
+
 // logits [n, V] float32; temperature [n] float32 or null (all greedy); seed, draws [n] int64.
 SOC_EXPORT int soc_sample(const float* logits, const float* temperature, const long long* seed,
                           const long long* draws, int* out, int n, int V, hipStream_t stream) {

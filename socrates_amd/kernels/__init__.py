@@ -51,7 +51,7 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
 }
-_SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P]}
+_SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
@@ -399,7 +399,15 @@ class HipKernels:
 
     # -- sampling ------------------------------------------------------------------------------
     def argmax(self, logits):
-        return self.sample(logits, None, None, None)
+        """Greedy tokens, the lowest index among equal maxima; int32 [n]."""
+        n, V = logits.shape
+        self._want(logits, "logits", torch.float32)
+        n_chunks = max(1, min(64, V // 2048))
+        partial = torch.empty((n, n_chunks, 2), dtype=torch.float32, device=self.device)
+        out = torch.empty((n,), dtype=torch.int32, device=self.device)
+        _check(self._sampling.soc_argmax(_ptr(logits), _ptr(partial), _ptr(out), c_int(n), c_int(V),
+                                         c_int(n_chunks), self._stream()), "argmax")
+        return out
 
     def sample(self, logits, temperature, seed, draws):
         """logits [n, V] float32; temperature [n] float32 (0: greedy), seed and draws [n] int64.
