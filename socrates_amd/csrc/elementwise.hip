@@ -70,20 +70,68 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const T* __rest
     }
 }
 
+// The same in one pass for rows of at most VPT * blockDim elements: a thread keeps its
+// elements in registers between the sum of squares and the scaling.
+template <typename T, int VPT>
+__global__ void add_rmsnorm_regs_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                                        const float* __restrict__ partials, int n_partials,
+                                        size_t partial_stride, const float* __restrict__ w,
+                                        T* __restrict__ out, const int* __restrict__ rows, int d, float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int n = rows ? rows[i] : i;
+    float* r = residual + (size_t)n * d;
+    const T* dl = delta ? delta + (size_t)n * d : nullptr;
+    const float* dp = partials ? partials + (size_t)n * d : nullptr;
+    float v[VPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+        const int j = threadIdx.x + u * blockDim.x;
+        v[u] = 0.f;
+        if (j < d) {
+            v[u] = r[j];
+            if (dl) v[u] += to_float(dl[j]);
+            if (dp) for (int s = 0; s < n_partials; ++s) v[u] += dp[s * partial_stride + j];
+            if (!rows && (dl || dp)) r[j] = v[u];
+        }
+        ss += v[u] * v[u];
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    T* o = out + (size_t)i * d;
+#pragma unroll
+    for (int u = 0; u < VPT; ++u) {
+        const int j = threadIdx.x + u * blockDim.x;
+        if (j < d) o[j] = from_float<T>(v[u] * inv * w[j]);
+    }
+}
+
+template <typename T>
+static void launch_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
+                               size_t partial_stride, const float* w, void* out, const int* rows, int n_out,
+                               int d, float eps, hipStream_t stream) {
+    constexpr int VPT = 8;
+    const int threads = d <= 1024 ? 128 : (d <= 2048 ? 256 : (d <= 4096 ? 512 : 1024));
+    if (d <= VPT * threads)
+        hipLaunchKernelGGL((add_rmsnorm_regs_kernel<T, VPT>), dim3(n_out), dim3(threads), 0, stream, residual,
+                           (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
+    else
+        hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(1024), 0, stream, residual, (const T*)delta,
+                           partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
+}
+
 SOC_EXPORT int soc_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
                                long long partial_stride, const float* w, void* out, const int* rows,
                                int n_out, int d, float eps, int dtype, hipStream_t stream) {
     if (n_out <= 0) return 0;
     if (delta && partials) return (int)hipErrorInvalidValue;
-    const int threads = d >= 2048 ? 512 : 256;
     if (dtype == 0)
-        hipLaunchKernelGGL(add_rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, stream, residual,
-                           (const float*)delta, partials, n_partials, (size_t)partial_stride, w,
-                           (float*)out, rows, d, eps);
+        launch_add_rmsnorm<float>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
+                                  n_out, d, eps, stream);
     else
-        hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, dim3(n_out), dim3(threads), 0, stream, residual,
-                           (const bf16*)delta, partials, n_partials, (size_t)partial_stride, w,
-                           (bf16*)out, rows, d, eps);
+        launch_add_rmsnorm<bf16>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
+                                 n_out, d, eps, stream);
     return soc_last_error();
 }
 

@@ -84,6 +84,10 @@ class HipKernels:
         self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
         self.attention_row_tiles = None     # row tiles per wave of the MFMA kernel, override
         self.attention_mfma = True          # bfloat16 takes the MFMA kernel
+        # bfloat16 products with more than 16 rows go to the library (hipBLASLt through
+        # torch.mm), as the reference's all do (nn.Linear); False keeps them on this
+        # package's tiled MFMA kernel
+        self.library_gemm = True
         self._decode_blocks = None
 
     # -- helpers -----------------------------------------------------------------------------
@@ -173,7 +177,9 @@ class HipKernels:
     # -- matrix products ------------------------------------------------------------------------
     def linear(self, x, w, out_dtype=None, allow_partial=False, row_tiles=0, n_waves=0, k_splits=0):
         """x [M, K] times w [N, K] transposed. float32 operands (either) take the plain
-        float32 kernel; bfloat16 pairs take the MFMA kernels. ``allow_partial``: the consumer
+        float32 kernel. bfloat16 pairs: up to 16 rows the skinny MFMA kernel (it streams
+        the weights faster than the library does there); more rows the library product,
+        or this package's tiled MFMA kernel if ``library_gemm`` is off. ``allow_partial``: the consumer
         (the residual-add + norm kernel) accepts float32 split-K partial sums [S, M, N]; the
         skinny kernel then spreads a narrow output over more workgroups."""
         self._want(x, "x")
@@ -187,7 +193,8 @@ class HipKernels:
         if M == 0:
             return torch.empty((M, N), dtype=out_dtype, device=self.device)
         both_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-        if both_bf16 and K % 8 == 0 and K >= 8 and M <= 64:
+        skinny_rows = 16 if self.library_gemm else 64
+        if both_bf16 and K % 8 == 0 and K >= 8 and M <= skinny_rows:
             if not (row_tiles and n_waves and k_splits):
                 rw, nw, ks = c_int(0), c_int(0), c_int(0)
                 self._gemm.soc_gemm_skinny_plan(c_int(M), c_int(N), c_int(K), c_int(1 if allow_partial else 0),
@@ -205,6 +212,10 @@ class HipKernels:
                                                    c_int(n_waves), c_int(k_splits), self._stream()),
                    f"linear [{M}x{K}] x [{N}x{K}]^T")
             return out
+        if both_bf16 and self.library_gemm:
+            if out_dtype == torch.bfloat16:
+                return torch.mm(x, w.t())
+            return torch.mm(x, w.t(), out_dtype=out_dtype)
         out = torch.empty((M, N), dtype=out_dtype, device=self.device)
         args = (_ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K))
         if both_bf16 and K % 8 == 0 and K >= 8:

@@ -46,7 +46,7 @@ def test_embedding(kernel_sets, dtype, N, V, d):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("N,d,eps", [(1, 64, 1e-6), (7, 72, 1e-5), (19, 2560, 1e-6), (3, 5000, 1e-2)])
+@pytest.mark.parametrize("N,d,eps", [(1, 64, 1e-6), (7, 72, 1e-5), (19, 2560, 1e-6), (3, 5000, 1e-2), (2, 9000, 1e-6)])
 def test_add_rmsnorm(kernel_sets, dtype, N, d, eps):
     hip, ref = kernel_sets[dtype]
     w = (1 + 0.3 * torch.randn(d)).to(DEV)
@@ -94,13 +94,16 @@ def test_swiglu(kernel_sets, dtype, N, ff):
 def test_linear(kernel_sets, a_dt, w_dt, c_dt, M, N, K):
     hip, _ = kernel_sets[a_dt]
     x, w = rnd((M, K), a_dt, 6), rnd((N, K), w_dt, 7, K ** -0.5)
-    got = hip.linear(x, w, out_dtype=c_dt)
     want = x.double() @ w.double().T
-    assert got.dtype == c_dt
-    if c_dt == torch.float32:
-        torch.testing.assert_close(got.double(), want, atol=3e-5, rtol=3e-5)
-    else:
-        torch.testing.assert_close(got.double(), want, atol=2e-2, rtol=2e-2)
+    for library in (True, False):        # the library product for many rows, and this package's kernels
+        hip.library_gemm = library
+        got = hip.linear(x, w, out_dtype=c_dt)
+        assert got.dtype == c_dt
+        if c_dt == torch.float32:
+            torch.testing.assert_close(got.double(), want, atol=3e-5, rtol=3e-5)
+        else:
+            torch.testing.assert_close(got.double(), want, atol=2e-2, rtol=2e-2)
+    hip.library_gemm = True
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (8, 2560, 9728), (40, 100, 2048), (64, 6144, 2560)])
@@ -110,6 +113,7 @@ def test_linear_split_k_partials(kernel_sets, M, N, K):
     hip, ref = kernel_sets[torch.bfloat16]
     x, w = rnd((M, K), torch.bfloat16, 6), rnd((N, K), torch.bfloat16, 7, K ** -0.5)
     want = x.double() @ w.double().T
+    hip.library_gemm = False            # this package's skinny kernel for every M up to 64
     for ks in (0, 1, 2, 4, 7):
         got = hip.linear(x, w, allow_partial=True, k_splits=ks)
         if ks > 1:
@@ -124,6 +128,7 @@ def test_linear_split_k_partials(kernel_sets, M, N, K):
             b = ref.add_rmsnorm(r2, got, gain, 1e-6)
             close(a, b, torch.bfloat16)
             torch.testing.assert_close(r1, r2, atol=1e-5, rtol=1e-5)
+    hip.library_gemm = True
 
 
 def test_linear_float32_is_not_reduced_precision(kernel_sets):
