@@ -588,4 +588,225 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     return soc_last_error();
 }
 
+
+// =============================================================================================
+// Prompt portions (bfloat16): a workgroup of four waves owns 4 * RT * 16 rows of one sequence
+// and kv head (consecutive tokens x the heads of the group) and walks the keys 32 at a time.
+// The four waves load each K and V tile once, together, into LDS (V transposed on the way,
+// so that a slice of V^T for the second product is one 8-byte read), which cuts the traffic
+// from L2 by four against one wave per row block. Tiles are double-buffered in LDS and the
+// next tile's global loads are issued before the current tile's products. Products, softmax
+// and layouts are those of paged_attn_mfma_kernel; the second product takes 32 keys per MFMA.
+constexpr int PF_KEYS = 32;
+constexpr int PF_K_STRIDE = D + 8;                  // K tile [32][D + 8]
+constexpr int PF_V_STRIDE = PF_KEYS + 4;            // V^T tile [D][32 + 4]
+constexpr int PF_CHUNKS = PF_KEYS * D / 8;          // 16-byte chunks per tile and operand
+constexpr int PF_PER_THREAD = (PF_CHUNKS + 255) / 256;
+constexpr int PF_K_ELEMS = PF_KEYS * PF_K_STRIDE, PF_V_ELEMS = D * PF_V_STRIDE;
+
+template <int RT>
+__global__ void __launch_bounds__(256)
+paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
+                          const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
+                          int table_width, const int* __restrict__ token_rows,
+                          const int* __restrict__ positions, const int* __restrict__ row_blocks,
+                          bf16* __restrict__ out, int Hq, int Hkv, int BS, float scale, int window,
+                          int group_pad_log2) {
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][PF_K_ELEMS];
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][PF_V_ELEMS];
+    const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
+    const int li = lane % 16, kb = lane / 16;
+    const int G = Hq / Hkv, Gp = 1 << group_pad_log2;
+    const int chunks = (G + 15) / 16;
+    const int blk = blockIdx.x / (Hkv * chunks);
+    const int kvh = (blockIdx.x / chunks) % Hkv, chunk = blockIdx.x % chunks;
+    const int tok0 = row_blocks[2 * blk], ntok = row_blocks[2 * blk + 1];
+    const int pos0 = positions[tok0];
+    const int* table = block_table + (size_t)token_rows[tok0] * table_width;
+    const int tokens_per_wave = (16 * RT) >> group_pad_log2;
+
+    const int khi = pos0 + ntok;                                    // keys any row of the block sees
+    const int kmin = window > 0 ? max(0, pos0 - window + 1) : 0;
+    const int klo = kmin & ~(PF_KEYS - 1);
+    // this wave's rows
+    const int wtok0 = wave * tokens_per_wave;                       // first token of the wave in the block
+    const int wave_hi = min(khi, pos0 + wtok0 + tokens_per_wave);   // keys past this are hidden from the wave
+    const bool wave_has_rows = wtok0 < ntok;
+
+    int row_pos[RT];
+    size_t row_q[RT];
+    uint4 qf[RT][QK_STEPS];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int rho = rt * 16 + li;
+        const int tt = wtok0 + (rho >> group_pad_log2), g = chunk * 16 + (rho & (Gp - 1));
+        const bool ok = tt < ntok && g < G;
+        row_pos[rt] = ok ? pos0 + tt : -1;
+        row_q[rt] = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? g : 0)) * D;
+#pragma unroll
+        for (int kk = 0; kk < QK_STEPS; ++kk)
+            qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
+    }
+    f32x4_t o[RT][DV];
+    float m[RT], l[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m[rt] = -INFINITY; l[rt] = 0.f;
+#pragma unroll
+        for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    }
+
+    // cooperative tile loads: thread -> chunks (key, part) of K and of V
+    uint4 kr[PF_PER_THREAD], vr[PF_PER_THREAD];
+    auto fetch = [&](int key0) {
+#pragma unroll
+        for (int j = 0; j < PF_PER_THREAD; ++j) {
+            const int c = tid + 256 * j;
+            const int ck = c / (D / 8), part = c % (D / 8);
+            const int key = key0 + ck;
+            if ((PF_CHUNKS % 256 == 0 || c < PF_CHUNKS) && key >= kmin && key < khi) {
+                const size_t off = ((size_t)table[key / BS] * Hkv * BS + (size_t)kvh * BS + key % BS) * D + part * 8;
+                kr[j] = *reinterpret_cast<const uint4*>(k_pool + off);
+                vr[j] = *reinterpret_cast<const uint4*>(v_pool + off);
+            } else {
+                kr[j] = make_uint4(0u, 0u, 0u, 0u);                  // unseen keys are never read
+                vr[j] = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < PF_PER_THREAD; ++j) {
+            const int c = tid + 256 * j;
+            if (PF_CHUNKS % 256 == 0 || c < PF_CHUNKS) {
+                const int ck = c / (D / 8), part = c % (D / 8);
+                *reinterpret_cast<uint4*>(&k_lds[buf][ck * PF_K_STRIDE + part * 8]) = kr[j];
+                const uint32_t w4[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
+                uint16_t* vt = &v_lds[buf][(part * 8) * PF_V_STRIDE + ck];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    vt[(2 * e) * PF_V_STRIDE] = (uint16_t)(w4[e] & 0xffffu);
+                    vt[(2 * e + 1) * PF_V_STRIDE] = (uint16_t)(w4[e] >> 16);
+                }
+            }
+        }
+    };
+
+    if (klo < khi) { fetch(klo); stash(0); }
+    __syncthreads();
+    int buf = 0;
+    for (int key0 = klo; key0 < khi; key0 += PF_KEYS) {
+        const bool more = key0 + PF_KEYS < khi;
+        if (more) fetch(key0 + PF_KEYS);
+        if (wave_has_rows && key0 < wave_hi) {
+            const uint16_t* kt = k_lds[buf];
+            const uint16_t* vt = v_lds[buf];
+            s16x4_t pf[RT][2];
+            float alpha[RT];
+            bool any_rescale = false;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                f32x4_t s0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+                for (int kk = 0; kk < QK_STEPS; ++kk) {
+                    const uint4 ka = load_qk_slice(reinterpret_cast<const bf16*>(kt + li * PF_K_STRIDE), kk, kb);
+                    const uint4 kc = load_qk_slice(reinterpret_cast<const bf16*>(kt + (16 + li) * PF_K_STRIDE), kk, kb);
+                    s0 = qk_mfma(ka, qf[rt][kk], s0);
+                    s1 = qk_mfma(kc, qf[rt][kk], s1);
+                }
+                float sv[8];
+                float mx = -INFINITY;
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    const int key = key0 + (r < 4 ? 0 : 16) + 4 * kb + (r & 3);
+                    bool seen = key <= row_pos[rt] && key < khi;
+                    if (window > 0) seen = seen && key > row_pos[rt] - window;
+                    sv[r] = seen ? (r < 4 ? s0[r & 3] : s1[r & 3]) * scale : -INFINITY;
+                    mx = fmaxf(mx, sv[r]);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
+                const float mn = fmaxf(m[rt], mx);
+                const float ms = mn == -INFINITY ? 0.f : mn;
+                alpha[rt] = __expf(m[rt] - ms);
+                float psum = 0.f;
+                uint16_t pb[8];
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    const float p = __expf(sv[r] - ms);
+                    psum += p;
+                    pb[r] = f32_to_bf16_bits(p);
+                }
+                l[rt] = l[rt] * alpha[rt] + psum;
+                any_rescale = any_rescale || (m[rt] != mn);
+                m[rt] = mn;
+                pf[rt][0] = (s16x4_t){(short)pb[0], (short)pb[1], (short)pb[2], (short)pb[3]};
+                pf[rt][1] = (s16x4_t){(short)pb[4], (short)pb[5], (short)pb[6], (short)pb[7]};
+            }
+            if (__any(any_rescale)) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
+            }
+#pragma unroll
+            for (int j = 0; j < DV; ++j) {
+                const uint16_t* src = vt + (j * 16 + li) * PF_V_STRIDE + 4 * kb;
+                const s16x4_t va = *reinterpret_cast<const s16x4_t*>(src);          // keys 4kb .. 4kb+3
+                const s16x4_t vc = *reinterpret_cast<const s16x4_t*>(src + 16);     // keys 16+4kb ..
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pf[rt][0], o[rt][j], 0, 0, 0);
+                    o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vc, pf[rt][1], o[rt][j], 0, 0, 0);
+                }
+            }
+        }
+        if (more) stash(buf ^ 1);           // the other buffer: nobody reads it in this iteration
+        __syncthreads();
+        buf ^= 1;
+    }
+
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float L = l[rt];
+        L += __shfl_xor(L, 16, SOC_WAVE);
+        L += __shfl_xor(L, 32, SOC_WAVE);
+        if (row_pos[rt] < 0) continue;
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
+#pragma unroll
+        for (int j = 0; j < DV; ++j) {
+            uint2 pk;
+            pk.x = (uint32_t)f32_to_bf16_bits(o[rt][j][0] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][1] * inv) << 16);
+            pk.y = (uint32_t)f32_to_bf16_bits(o[rt][j][2] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][3] * inv) << 16);
+            *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
+        }
+    }
+}
+
+// bfloat16 only, no key splits. row_blocks [n_row_blocks, 2] = (first token, tokens) of each
+// block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of one sequence.
+SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
+                                           const int* block_table, int table_width, const int* token_rows,
+                                           const int* positions, const int* row_blocks, int n_row_blocks,
+                                           void* out, int N, int Hq, int Hkv, int BS, float scale,
+                                           int window, int row_tiles, int group_pad_log2,
+                                           hipStream_t stream) {
+    if (N <= 0 || n_row_blocks <= 0) return 0;
+    if (Hkv < 1 || Hq % Hkv || BS < 1) return (int)hipErrorInvalidValue;
+    const int G = Hq / Hkv;
+    if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
+    const long groups = (long)n_row_blocks * Hkv * ((G + 15) / 16);
+    if (groups > 0x7fffffffL) return (int)hipErrorInvalidValue;
+#define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
+        token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, scale, window, group_pad_log2
+    if (row_tiles == 1)
+        hipLaunchKernelGGL(paged_attn_prefill_kernel<1>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+    else if (row_tiles == 2)
+        hipLaunchKernelGGL(paged_attn_prefill_kernel<2>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+    else
+        return (int)hipErrorInvalidValue;
+#undef SOC_PF_ARGS
+    return soc_last_error();
+}
+
 SOC_EXPORT int soc_attention_head_dim() { return D; }

@@ -55,6 +55,7 @@ _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
+    "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
     "soc_attention_head_dim": [],
 }
 
@@ -83,7 +84,8 @@ class HipKernels:
         _declare(self._sampling, _SAMPLING_SIGNATURES)
         self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
         self.attention_row_tiles = None     # row tiles per wave of the MFMA kernel, override
-        self.attention_mfma = True          # bfloat16 takes the MFMA kernel
+        self.attention_mfma = True          # bfloat16 takes the MFMA kernels
+        self.attention_workgroup = True     # prompt portions take the kernel that shares K/V through LDS
         # bfloat16 products with more than 16 rows go to the library (hipBLASLt through
         # torch.mm), as the reference's all do (nn.Linear); False keeps them on this
         # package's tiled MFMA kernel
@@ -372,6 +374,20 @@ class HipKernels:
         if self.dtype == torch.bfloat16 and self.attention_mfma:
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
+            if N > 65535:
+                raise KernelError("more than 65535 tokens in one attention call")
+            if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
+                    and getattr(ctx, "max_q_len", 1) >= 16):
+                # prompt portions: four waves of a workgroup share the K and V tiles
+                rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2) else (2 if D <= 64 else 1)
+                blocks, n_blocks = self._row_blocks(ctx, N, 4 * max(1, (16 * rt) >> gpl))
+                _check(lib.soc_paged_attention_prefill(
+                    _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+                    c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
+                    c_int(n_blocks), _ptr(out), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
+                    c_float(scale), c_int(w), c_int(rt), c_int(gpl), self._stream()),
+                    "paged_attention (prefill)")
+                return out
             rt = self.attention_row_tiles or (1 if decode else 2 if D <= 128 else 1)
             tokens_per_block = max(1, (16 * rt) >> gpl)
             blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
@@ -380,8 +396,6 @@ class HipKernels:
             if n_splits > 1:
                 part_o = torch.empty((N, Hq, n_splits, D), dtype=torch.float32, device=self.device)
                 part_ml = torch.empty((N, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
-            if N > 65535:
-                raise KernelError("more than 65535 tokens in one attention call")
             _check(lib.soc_paged_attention_mfma(
                 _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
                 c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),

@@ -225,11 +225,32 @@ def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     q = rnd((len(rows), Hq, D), dtype, 9)
     for window in (None, 1, 7, 16, 64):
         want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
-        for row_tiles, splits in ((None, None), (1, (32, 5)), (2, None), (4, (64, 3)), (4, None)):
-            hip.attention_row_tiles, hip.attention_splits = row_tiles, splits
+        # (row tiles, splits, workgroup kernel): the per-wave and the workgroup MFMA kernels
+        for row_tiles, splits, wg in ((None, None, True), (1, None, True), (2, None, True), (1, (32, 5), False),
+                                      (2, None, False), (4, (64, 3), False), (4, None, False)):
+            hip.attention_row_tiles, hip.attention_splits, hip.attention_workgroup = row_tiles, splits, wg
             got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
             close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
     hip.attention_row_tiles = hip.attention_splits = None
+    hip.attention_workgroup = True
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,bs", [(4, 2, 16, 16), (9, 3, 48, 4), (32, 8, 128, 16), (16, 1, 64, 32), (40, 2, 32, 8)])
+def test_prefill_attention_whole_prompts(kernel_sets, Hq, Hkv, D, bs):
+    """Whole prompts and long portions through the workgroup kernel: several sequences of
+    uneven length, one of them continuing a cache of 100 tokens."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    lens = [257, 33, 100 + 75, 16]
+    slot, dense = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=D + 1)
+    rows = [0] * 257 + [1] * 33 + [2] * 75 + [3] * 16
+    pos = list(range(257)) + list(range(33)) + list(range(100, 175)) + list(range(16))
+    q = rnd((len(rows), Hq, D), torch.bfloat16, 21)
+    want = dense_attention(q, dense, rows, pos, D ** -0.5)
+    for rt in (1, 2):
+        hip.attention_row_tiles = rt
+        got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5)
+        close(got.cpu(), want, torch.bfloat16)
+    hip.attention_row_tiles = None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
