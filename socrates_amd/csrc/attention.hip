@@ -526,25 +526,20 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
     float M = -INFINITY;
     for (int s = lane; s < n_splits; s += SOC_WAVE) M = fmaxf(M, part_ml[(base + s) * 2]);
     M = wave_max(M);
-    float L = 0.f;
-    for (int s0 = 0; s0 < n_splits; s0 += 256) {           // weights of up to 256 splits at a time
-        float lsum = 0.f;
-        for (int s = s0 + lane; s < min(n_splits, s0 + 256); s += SOC_WAVE) {
-            const float ms = part_ml[(base + s) * 2];
-            const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
-            weight[s - s0] = w;
-            lsum += w * part_ml[(base + s) * 2 + 1];
-        }
-        L += wave_sum(lsum);
-        if (s0 + 256 < n_splits) break;                     // (more than 256 splits: handled below)
+    float lsum = 0.f;                                       // the launcher allows at most 256 splits
+    for (int s = lane; s < n_splits; s += SOC_WAVE) {
+        const float ms = part_ml[(base + s) * 2];
+        const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+        weight[s] = w;
+        lsum += w * part_ml[(base + s) * 2 + 1];
     }
+    const float L = wave_sum(lsum);
     __syncthreads();
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    const int first = min(n_splits, 256);
     for (int e = lane; e < D; e += SOC_WAVE) {
         float A = 0.f;
 #pragma unroll 4
-        for (int s = 0; s < first; ++s) A += part_o[(base + s) * D + e] * weight[s];
+        for (int s = 0; s < n_splits; ++s) A += part_o[(base + s) * D + e] * weight[s];
         out[((size_t)n * Hq + h) * D + e] = from_float<bf16>(A * inv);
     }
 }

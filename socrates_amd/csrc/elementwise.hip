@@ -166,30 +166,42 @@ SOC_EXPORT int soc_rmsnorm(const void* x, const float* w, void* out, int R, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[n, j] = silu(gate_up[n, j]) * gate_up[n, ff + j],  silu(z) = z / (1 + exp(-z))
+// out[n, j] = silu(gate[n, j]) * up[n, j],  silu(z) = z / (1 + exp(-z)). gate_up holds
+// [gate | up] halves (interleave 0), or gate and up columns alternating in blocks of
+// `interleave` (the layout of a fused weight whose rows alternate that way).
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff) {
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, size_t total, int ff,
+                              int interleave) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < total; i += stride) {
         const size_t n = i / ff, j = i % ff;
-        const float g = to_float(gate_up[n * 2 * ff + j]);
-        const float u = to_float(gate_up[n * 2 * ff + ff + j]);
+        size_t gi, ui;
+        if (interleave > 0) {
+            gi = (j / interleave) * 2 * interleave + j % interleave;
+            ui = gi + interleave;
+        } else {
+            gi = j; ui = ff + j;
+        }
+        const float g = to_float(gate_up[n * 2 * ff + gi]);
+        const float u = to_float(gate_up[n * 2 * ff + ui]);
         out[i] = from_float<T>(u * (g / (1.0f + expf(-g))));
     }
 }
 
-SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int dtype, hipStream_t stream) {
+SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int interleave, int dtype,
+                          hipStream_t stream) {
     const size_t total = (size_t)N * ff;
     if (total == 0) return 0;
+    if (interleave < 0 || (interleave > 0 && ff % interleave)) return (int)hipErrorInvalidValue;
     size_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
     if (dtype == 0)
         hipLaunchKernelGGL(swiglu_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           (const float*)gate_up, (float*)out, total, ff);
+                           (const float*)gate_up, (float*)out, total, ff, interleave);
     else
         hipLaunchKernelGGL(swiglu_kernel<bf16>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           (const bf16*)gate_up, (bf16*)out, total, ff);
+                           (const bf16*)gate_up, (bf16*)out, total, ff, interleave);
     return soc_last_error();
 }
 

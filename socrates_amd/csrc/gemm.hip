@@ -4,13 +4,15 @@
 //  gemm_generic_kernel   any sizes and any mix of float32 / bfloat16 operands; plain FMA in
 //                        float32, K summed in order. This is the true 32-bit path.
 //  gemm_bf16_mfma_kernel bfloat16 operands, 128x128x64 tiles through LDS, 16x16x32 MFMA with
-//                        float32 accumulators: prompt portions (large M).
-//  gemm_bf16_skinny_kernel bfloat16, M <= 64 (decode): bound by streaming W once from HBM. A
-//                        workgroup owns 16 rows of W, its waves split K, every lane keeps
-//                        several 16-byte loads of W in flight, the weights are the MFMA's
-//                        first operand so that one lane ends up with four consecutive
-//                        outputs; the waves' partial tiles are summed through LDS in a fixed
-//                        order.
+//                        float32 accumulators. The library's product is faster for many rows
+//                        and is what the engine uses there; this kernel stays as the
+//                        package's own path (HipKernels.library_gemm = False).
+//  gemm_bf16_skinny_kernel bfloat16, M <= 64 (the engine uses it up to 16 rows: decode). Bound
+//                        by streaming W once from HBM: 16-byte slices of 16 weight rows per
+//                        wave load, two buffers in flight, weights as the MFMA's first
+//                        operand so that one lane ends up with four consecutive outputs,
+//                        optional split of K over workgroups (float32 partial sums) and an
+//                        optional SwiGLU epilogue.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -208,7 +210,10 @@ constexpr int SK_MAX_WAVES = 8;
 
 template <int MT, int RW> struct SkBuf { uint4 w[RW][SK_UNROLL]; uint4 x[MT][SK_UNROLL]; };
 
-template <typename TC, int MT, int RW>
+// SWIGLU: the two row tiles of a workgroup are 16 gate rows and the 16 up rows of the same
+// output columns (the weight's rows are interleaved in blocks of 16); the epilogue writes
+// silu(gate) * up, [M, N / 2], instead of both products.
+template <typename TC, int MT, int RW, bool SWIGLU = false>
 __global__ void __launch_bounds__(64 * SK_MAX_WAVES)
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
@@ -310,6 +315,20 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
             for (int e = 0; e < 4; ++e)
                 red[(((wave * MT + t) * RW + r) * 64 + lane) * 4 + e] = acc[t][r][e];
     __syncthreads();
+    if constexpr (SWIGLU) {
+        static_assert(!SWIGLU || RW == 2, "gate and up tiles");
+        for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
+            const int t = idx / 256, ln = (idx % 256) / 4, e = idx % 4;
+            float g = 0.f, u = 0.f;
+            for (int w = 0; w < n_waves; ++w) {
+                g += red[(((w * MT + t) * RW + 0) * 64 + ln) * 4 + e];
+                u += red[(((w * MT + t) * RW + 1) * 64 + ln) * 4 + e];
+            }
+            const int m = t * 16 + ln % 16, col = blockIdx.x * 16 + 4 * (ln / 16) + e;
+            if (m < M && 2 * col < N) C[(size_t)m * (N / 2) + col] = from_float<TC>(u * (g / (1.0f + expf(-g))));
+        }
+        return;
+    }
     for (int idx = tid; idx < MT * RW * 256; idx += blockDim.x) {
         const int tr = idx / 256, ln = (idx % 256) / 4, e = idx % 4;
         const int t = tr / RW, r = tr % RW;
@@ -332,6 +351,26 @@ static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, in
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT, RW>), dim3((N + 16 * RW - 1) / (16 * RW), k_splits),
                        dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (TC*)C, Cpart, M, N,
                        K, k_per_split, k_per_wave);
+    return soc_last_error();
+}
+
+// x [M <= 16, K] times w [N, K]^T with gate and up rows interleaved in blocks of 16, then
+// silu(gate) * up: C [M, N / 2]. N a multiple of 32, K a multiple of 8.
+SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C, int M, int N, int K,
+                                           int c_dtype, int n_waves, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 || K < 8 || N % 32) return (int)hipErrorInvalidValue;
+    if (n_waves < 1 || n_waves > SK_MAX_WAVES) return (int)hipErrorInvalidValue;
+    const int k_per_wave = ((K + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
+    const int k_per_split = k_per_wave * n_waves;
+    if (c_dtype == 0)
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 2, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+                           stream, (const bf16*)X, (const bf16*)W, (float*)C, (float*)nullptr, M, N, K,
+                           k_per_split, k_per_wave);
+    else
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 2, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+                           stream, (const bf16*)X, (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K,
+                           k_per_split, k_per_wave);
     return soc_last_error();
 }
 

@@ -73,8 +73,8 @@ class ModelRunner:
     # is replayed from a graph captured for its width (rounded up to a bucket; the padding
     # rows use the cache's null row, so they read and write the null page only). The graph's
     # inputs live at fixed addresses and are filled by one copy per step; key splits of the
-    # attention kernel are planned for the longest context the cache allows, so the launch
-    # shape never depends on a request's length.
+    # attention kernel are planned for a bucket of context lengths (powers of two), so the
+    # launch shape depends on a request's length only through that bucket.
     _BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 
     def enable_graphs(self, max_width: int) -> None:
@@ -89,7 +89,15 @@ class ModelRunner:
                 return min(b, max(self._graph_max, n))
         return n
 
-    def _capture(self, width: int):
+    def _context_bucket(self, longest: int) -> int:
+        """The context length a graph is planned for: the next power of two (at least 256),
+        capped by the cache's longest row."""
+        b = 256
+        while b < longest:
+            b *= 2
+        return min(b, self.cache.max_len)
+
+    def _capture(self, width: int, context: int):
         dev = self.ops.device
         inputs = torch.zeros((3, width), dtype=torch.int32, device=dev)
         inputs[2].fill_(self.cache.null_row)
@@ -98,7 +106,7 @@ class ModelRunner:
         ctx = StepContext(
             n_tokens=width, n_seqs=width, n_want=width, token_ids=inputs[0], positions=inputs[1],
             token_rows=inputs[2], seq_rows=inputs[2], seq_qstart=arange, seq_ctx=inputs[1],
-            want_index=arange[:width], max_q_len=1, max_ctx_len=self.cache.max_len, host={})
+            want_index=arange[:width], max_q_len=1, max_ctx_len=context, host={})
         stream = torch.cuda.Stream(device=dev)
         stream.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(stream):
@@ -119,9 +127,13 @@ class ModelRunner:
         if len(set(rows)) != n:
             raise ValueError("a cache row appears twice in one step")
         width = self._bucket(n)
-        if width not in self._graphs:
-            self._graphs[width] = self._capture(width)
-        graph, inputs, staging, logits, _ctx = self._graphs[width]
+        # key splits of the attention kernel are planned per context bucket, so that a short
+        # context is not cut into the many splits a long one needs
+        context = self._context_bucket(max(cache.length(r) for r in rows) + 1)
+        key = (width, context)
+        if key not in self._graphs:
+            self._graphs[key] = self._capture(width, context)
+        graph, inputs, staging, logits, _ctx = self._graphs[key]
         host = staging.numpy()
         host[0, n:], host[1, n:], host[2, n:] = 0, 0, cache.null_row
         for i, e in enumerate(entries):

@@ -40,7 +40,7 @@ _EW_SIGNATURES = {
     "soc_embedding": [P, P, P, I, I, I, I, P],
     "soc_add_rmsnorm": [P, P, P, I, c_longlong, P, P, P, I, I, F, I, P],
     "soc_rmsnorm": [P, P, P, I, I, F, I, P],
-    "soc_swiglu": [P, P, I, I, I, P],
+    "soc_swiglu": [P, P, I, I, I, I, P],
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
     "soc_rope": [P, P, P, I, I, I, I, I, P],
     "soc_kv_write": [P] * 5 + [I, P, P, I, I, I, I, I, P],
@@ -50,6 +50,7 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_mfma": [P, P, P, I, I, I, I, P],
     "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
+    "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -166,15 +167,36 @@ class HipKernels:
                                     c_float(eps), c_int(self.code), self._stream()), "rmsnorm")
         return out
 
-    def swiglu(self, gate_up):
+    def swiglu(self, gate_up, interleave=0):
+        """silu(gate) * up from a [N, 2 ff] tensor holding [gate | up] (interleave 0) or gate and
+        up columns alternating in blocks of ``interleave``."""
         self._want(gate_up, "gate_up", self.dtype)
         N, two_ff = gate_up.shape
-        if two_ff % 2:
-            raise KernelError("gate_up needs an even last dimension")
+        if two_ff % 2 or (interleave and (two_ff // 2) % interleave):
+            raise KernelError("gate_up needs an even last dimension that the interleave divides")
         out = torch.empty((N, two_ff // 2), dtype=self.dtype, device=self.device)
-        _check(self._ew.soc_swiglu(_ptr(gate_up), _ptr(out), c_int(N), c_int(two_ff // 2),
+        _check(self._ew.soc_swiglu(_ptr(gate_up), _ptr(out), c_int(N), c_int(two_ff // 2), c_int(interleave),
                                    c_int(self.code), self._stream()), "swiglu")
         return out
+
+    def linear_swiglu(self, x, w_gate_up, interleave=0):
+        """swiglu(x @ w_gate_up^T). With rows interleaved in blocks of 16 and at most 16 rows of
+        x in bfloat16, one kernel: the skinny product applies silu(gate) * up in its epilogue."""
+        M, K = x.shape
+        N = w_gate_up.shape[0]
+        if (interleave == 16 and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N % 32 == 0):
+            self._want(x, "x")
+            self._want(w_gate_up, "weight", None, (N, K))
+            out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
+            n_waves = 8
+            while n_waves > 1 and K // n_waves < 128:
+                n_waves //= 2
+            _check(self._gemm.soc_gemm_bf16_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(N),
+                                                          c_int(K), c_int(self.code), c_int(n_waves),
+                                                          self._stream()), "linear_swiglu")
+            return out
+        return self.swiglu(self.linear(x, w_gate_up), interleave)
 
     # -- matrix products ------------------------------------------------------------------------
     def linear(self, x, w, out_dtype=None, allow_partial=False, row_tiles=0, n_waves=0, k_splits=0):
@@ -376,11 +398,17 @@ class HipKernels:
             decode = getattr(ctx, "max_q_len", 1) == 1
             if N > 65535:
                 raise KernelError("more than 65535 tokens in one attention call")
+            wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2) else (2 if D <= 64 else 1)
+            wg_tokens = 4 * max(1, (16 * wg_rt) >> gpl)
+            # Prompt portions go to the kernel whose four waves share the K and V tiles, if its
+            # workgroups fill the GPU (it has no key splits); a short portion behind a long
+            # context is better served by the per-wave kernel with key splits. An override of
+            # the row tiles (tests) forces the choice.
+            enough = (N // wg_tokens) * Hkv * ((G + 15) // 16) >= 512 or self.attention_row_tiles is not None
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
-                    and getattr(ctx, "max_q_len", 1) >= 16):
-                # prompt portions: four waves of a workgroup share the K and V tiles
-                rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2) else (2 if D <= 64 else 1)
-                blocks, n_blocks = self._row_blocks(ctx, N, 4 * max(1, (16 * rt) >> gpl))
+                    and getattr(ctx, "max_q_len", 1) >= 16 and enough):
+                rt = wg_rt
+                blocks, n_blocks = self._row_blocks(ctx, N, wg_tokens)
                 _check(lib.soc_paged_attention_prefill(
                     _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
                     c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
@@ -388,7 +416,7 @@ class HipKernels:
                     c_float(scale), c_int(w), c_int(rt), c_int(gpl), self._stream()),
                     "paged_attention (prefill)")
                 return out
-            rt = self.attention_row_tiles or (1 if decode else 2 if D <= 128 else 1)
+            rt = self.attention_row_tiles or 1
             tokens_per_block = max(1, (16 * rt) >> gpl)
             blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
             split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)

@@ -18,15 +18,23 @@ class SwiGLU:
 
     def __init__(self, spec: SwiGLUSpec, tensors, ops):
         self.spec, self.ops = spec, ops
-        # One operand for gate and up: rows [gate | up].
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]],
-                                   dim=0).contiguous()
+        # One operand for gate and up. Where the width allows, their rows alternate in blocks
+        # of 16 (16 gate rows, the 16 up rows of the same columns, ...): a workgroup of the
+        # decode product then holds both and applies the activation itself.
+        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        ff = spec.intermediate
+        self.interleave = 16 if ff % 16 == 0 else 0
+        if self.interleave:
+            self.w_gate_up = torch.stack([gate.view(ff // 16, 16, -1), up.view(ff // 16, 16, -1)],
+                                         dim=1).reshape(2 * ff, -1).contiguous()
+        else:
+            self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, x, ctx=None):
-        gate_up = self.ops.linear(x, self.w_gate_up)
+        act = self.ops.linear_swiglu(x, self.w_gate_up, self.interleave)
         # the block's next norm adds this output to the residual: partial sums are welcome
-        return self.ops.linear(self.ops.swiglu(gate_up), self.w_down, allow_partial=True)
+        return self.ops.linear(act, self.w_down, allow_partial=True)
 
 
 register_part(SwiGLUSpec, SwiGLU)

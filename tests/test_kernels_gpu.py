@@ -83,6 +83,24 @@ def test_swiglu(kernel_sets, dtype, N, ff):
     zero_gate = gu.clone()
     zero_gate[:, :ff] = 0
     assert hip.swiglu(zero_gate).abs().max() == 0       # silu is on the gate half
+    if ff % 16 == 0:
+        # the same with gate and up columns alternating in blocks of 16
+        mixed = torch.stack([gu[:, :ff].reshape(N, ff // 16, 16), gu[:, ff:].reshape(N, ff // 16, 16)], 2).reshape(N, 2 * ff)
+        close(hip.swiglu(mixed.contiguous(), 16), want, dtype)
+
+
+@pytest.mark.parametrize("M,ff,K", [(1, 128, 64), (8, 9728, 2560), (16, 160, 96), (5, 48, 256)])
+def test_linear_swiglu_fused(kernel_sets, M, ff, K):
+    """One kernel for the gate and up products and the activation (rows interleaved by 16)."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    x = rnd((M, K), torch.bfloat16, 30)
+    gate, up = rnd((ff, K), torch.bfloat16, 31, K ** -0.5), rnd((ff, K), torch.bfloat16, 32, K ** -0.5)
+    w = torch.stack([gate.view(ff // 16, 16, K), up.view(ff // 16, 16, K)], 1).reshape(2 * ff, K).contiguous()
+    want = torch.nn.functional.silu(x.float() @ gate.float().T) * (x.float() @ up.float().T)
+    close(hip.linear_swiglu(x, w, 16), want, torch.bfloat16)
+    big = rnd((40, K), torch.bfloat16, 33)                # more rows: product, then the activation kernel
+    want = torch.nn.functional.silu(big.float() @ gate.float().T) * (big.float() @ up.float().T)
+    close(hip.linear_swiglu(big, w, 16), want, torch.bfloat16)
 
 
 @pytest.mark.parametrize("a_dt,w_dt,c_dt", [

@@ -55,10 +55,18 @@ class TorchKernels:
     def rmsnorm(self, x, weight, eps):
         return self._norm(x, weight, eps).to(x.dtype)
 
-    def swiglu(self, gate_up):
+    def swiglu(self, gate_up, interleave=0):
         ff = gate_up.shape[-1] // 2
-        g, u = gate_up[..., :ff].to(self.acc), gate_up[..., ff:].to(self.acc)
+        if interleave:
+            blocks = gate_up.reshape(*gate_up.shape[:-1], ff // interleave, 2, interleave)
+            g, u = blocks[..., 0, :].reshape(*gate_up.shape[:-1], ff), blocks[..., 1, :].reshape(*gate_up.shape[:-1], ff)
+        else:
+            g, u = gate_up[..., :ff], gate_up[..., ff:]
+        g, u = g.to(self.acc), u.to(self.acc)
         return (u * (g * torch.sigmoid(g))).to(self.dtype)
+
+    def linear_swiglu(self, x, w_gate_up, interleave=0):
+        return self.swiglu(self.linear(x, w_gate_up), interleave)
 
     def linear(self, x, w, out_dtype=None, allow_partial=False):
         y = x.to(self.acc) @ w.to(self.acc).T
