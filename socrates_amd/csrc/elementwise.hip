@@ -189,11 +189,47 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
     }
 }
 
+// Eight columns per thread with 16-byte loads (bfloat16) when the layout allows: ff and the
+// interleave block are multiples of 8, so eight consecutive outputs share one gate run and
+// one up run.
+__global__ void swiglu_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, size_t groups,
+                                     int ff, int interleave) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const int per_row = ff / 8;
+    for (; i < groups; i += stride) {
+        const size_t n = i / per_row;
+        const int j = (int)(i % per_row) * 8;
+        size_t gi, ui;
+        if (interleave > 0) { gi = (size_t)(j / interleave) * 2 * interleave + j % interleave; ui = gi + interleave; }
+        else { gi = j; ui = (size_t)ff + j; }
+        float g[8], u[8];
+        VecLoad<bf16, 8>::load(gate_up + n * 2 * ff + gi, g);
+        VecLoad<bf16, 8>::load(gate_up + n * 2 * ff + ui, u);
+        uint32_t pk[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = u[2 * e] * (g[2 * e] / (1.0f + expf(-g[2 * e])));
+            const float b = u[2 * e + 1] * (g[2 * e + 1] / (1.0f + expf(-g[2 * e + 1])));
+            pk[e] = (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+        }
+        *reinterpret_cast<uint4*>(out + n * ff + j) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+    }
+}
+
 SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int interleave, int dtype,
                           hipStream_t stream) {
     const size_t total = (size_t)N * ff;
     if (total == 0) return 0;
     if (interleave < 0 || (interleave > 0 && ff % interleave)) return (int)hipErrorInvalidValue;
+    if (dtype == 1 && ff % 8 == 0 && interleave % 8 == 0) {
+        const size_t groups = total / 8;
+        size_t vblocks = (groups + 255) / 256;
+        if (vblocks > 65536) vblocks = 65536;
+        hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3((unsigned)vblocks), dim3(256), 0, stream,
+                           (const bf16*)gate_up, (bf16*)out, groups, ff, interleave);
+        return soc_last_error();
+    }
     size_t blocks = (total + 255) / 256;
     if (blocks > 16384) blocks = 16384;
     if (dtype == 0)
@@ -210,11 +246,13 @@ SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int int
 // (q and k only, if gains are given), rotate-half rotation at the token's position (q and k
 // only, if inv_freq is given), then store: q to q_out; k and v into the cache pages of the
 // token's row at its position, or to k_out / v_out when no pools are given.
-// One wave per head: workgroup (token, group of 4 heads), no loop, so a decode step's few
-// tokens still spread over many workgroups and the kernel is one short pass.
+// One wave per head. A workgroup of four waves takes 4 * heads_per_wave heads of one token:
+// one head per wave for a decode step (few tokens: many small workgroups, one short pass),
+// all heads of the token for prompt portions (fewer, fatter workgroups). A lane owns VE
+// consecutive elements of the head (VE = 2 at head size 128: one 4-byte access).
 #define SOC_MAX_HEAD 256
 
-template <typename T>
+template <typename T, int VE>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                     T* __restrict__ k_out, T* __restrict__ v_out,
@@ -224,71 +262,115 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                     const int* __restrict__ positions,
                                     const float* __restrict__ q_gain, const float* __restrict__ k_gain,
                                     const float* __restrict__ inv_freq, int Hq, int Hkv, int D,
-                                    int rotary_dim, int BS, float eps) {
-    __shared__ float stage[4][SOC_MAX_HEAD];
+                                    int rotary_dim, int BS, float eps, int heads_per_wave) {
+    __shared__ float cos_t[SOC_MAX_HEAD / 2], sin_t[SOC_MAX_HEAD / 2];
     const int n = blockIdx.x;
     const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
     const int heads = Hq + 2 * Hkv;
-    const int h = blockIdx.y * 4 + wave;
-    const bool active = h < heads;
-    const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
-    const T* x = qkv + ((size_t)n * heads + (active ? h : 0)) * D;
     const int pos = positions ? positions[n] : 0;
     const int half = rotary_dim / 2;
-    float v[SOC_MAX_HEAD / SOC_WAVE];
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-        const int e = lane + i * SOC_WAVE;
-        v[i] = e < D ? to_float(x[e]) : 0.f;
-        ss += v[i] * v[i];
-    }
-    const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
-    if (gain && active) {
-        ss = wave_sum(ss);
-        const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-#pragma unroll
-        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-            const int e = lane + i * SOC_WAVE;
-            if (e < D) v[i] = v[i] * inv * gain[e];
-        }
-    }
-    if (inv_freq) {                                   // uniform over the workgroup
-#pragma unroll
-        for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-            const int e = lane + i * SOC_WAVE;
-            if (e < D) stage[wave][e] = v[i];
-        }
+    const int e0 = lane * VE;                          // this lane's elements e0 .. e0 + VE - 1
+    const bool lane_on = e0 < D;                       // D is a multiple of VE
+    if (inv_freq) {
+        // the token's angles once per workgroup (float32, accurate range reduction:
+        // positions reach thousands of radians)
+        if ((int)threadIdx.x < half) sincosf((float)pos * inv_freq[threadIdx.x], &sin_t[threadIdx.x], &cos_t[threadIdx.x]);
         __syncthreads();
-        if (active && (is_q || is_k)) {
+    }
+    size_t page_base = 0;
+    if (k_pool) {
+        const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
+        page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;
+    }
+    // Heads are taken HB at a time per wave (their loads are issued together). Measured on
+    // prompt portions of 2,048 tokens, one at a time is as fast as four.
+    constexpr int HB = 1;
+    for (int it0 = 0; it0 < heads_per_wave; it0 += HB) {          // the same trip count for all waves
+        float vv[HB][VE];
 #pragma unroll
-            for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-                const int e = lane + i * SOC_WAVE;
-                if (e < rotary_dim) {
-                    const int j = e < half ? e : e - half;
-                    const float partner = stage[wave][e < half ? e + half : e - half];
-                    float sn, cs;
-                    sincosf((float)pos * inv_freq[j], &sn, &cs);
-                    v[i] = e < half ? v[i] * cs - partner * sn : v[i] * cs + partner * sn;
+        for (int b = 0; b < HB; ++b) {
+            const int h = (blockIdx.y * heads_per_wave + it0 + b) * 4 + wave;
+            const bool on = it0 + b < heads_per_wave && h < heads && lane_on;
+            if (on) VecLoad<T, VE>::load(qkv + ((size_t)n * heads + h) * D + e0, vv[b]);
+            else {
+#pragma unroll
+                for (int i = 0; i < VE; ++i) vv[b][i] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < HB; ++b) {
+            if (it0 + b >= heads_per_wave) break;                   // uniform
+            const int h = (blockIdx.y * heads_per_wave + it0 + b) * 4 + wave;
+            const bool active = h < heads;
+            const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
+            float (&v)[VE] = vv[b];
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < VE; ++i) ss += v[i] * v[i];
+            const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+            if (gain && active) {
+                ss = wave_sum(ss);
+                const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+                for (int i = 0; i < VE; ++i) if (lane_on) v[i] = v[i] * inv * gain[e0 + i];
+            }
+            if (inv_freq) {                                 // uniform over the wave
+                // the partner of element e is e +- half: the same slot of the lane half / VE away
+                // (half is a multiple of VE, checked by the launcher)
+                const int shift = half / VE;
+                const int src = e0 < half ? lane + shift : lane - shift;
+#pragma unroll
+                for (int i = 0; i < VE; ++i) {
+                    const float partner = __shfl(v[i], src & (SOC_WAVE - 1), SOC_WAVE);
+                    const int e = e0 + i;
+                    if (active && (is_q || is_k) && lane_on && e < rotary_dim) {
+                        const int j = e < half ? e : e - half;
+                        const float sn = sin_t[j], cs = cos_t[j];
+                        v[i] = e < half ? v[i] * cs - partner * sn : v[i] * cs + partner * sn;
+                    }
                 }
+            }
+            if (!active || !lane_on) continue;
+            T* dst;
+            if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
+            else {
+                const int kvh = is_k ? h - Hq : h - Hq - Hkv;
+                if (k_pool) dst = (is_k ? k_pool : v_pool) + page_base + (size_t)kvh * BS * D;
+                else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
+            }
+            if constexpr (VE == 1) {
+                dst[e0] = from_float<T>(v[0]);
+            } else if constexpr (sizeof(T) == 2) {
+                uint32_t pk[VE / 2];
+#pragma unroll
+                for (int i = 0; i < VE / 2; ++i)
+                    pk[i] = (uint32_t)f32_to_bf16_bits(v[2 * i]) | ((uint32_t)f32_to_bf16_bits(v[2 * i + 1]) << 16);
+                if constexpr (VE == 2) *reinterpret_cast<uint32_t*>(dst + e0) = pk[0];
+                else *reinterpret_cast<uint2*>(dst + e0) = make_uint2(pk[0], pk[1]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < VE; ++i) dst[e0 + i] = from_float<T>(v[i]);
             }
         }
     }
-    if (!active) return;
-    T* dst;
-    if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
-    else {
-        const int kvh = is_k ? h - Hq : h - Hq - Hkv;
-        if (k_pool) {
-            const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
-            dst = (is_k ? k_pool : v_pool) + (((size_t)page * Hkv + kvh) * BS + (size_t)(pos % BS)) * D;
-        } else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
-    }
-#pragma unroll
-    for (int i = 0; i < SOC_MAX_HEAD / SOC_WAVE; ++i) {
-        const int e = lane + i * SOC_WAVE;
-        if (e < D) dst[e] = from_float<T>(v[i]);
-    }
+}
+
+template <typename T>
+static void launch_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void* v_out, void* k_pool,
+                                void* v_pool, const int* block_table, int table_width,
+                                const int* token_rows, const int* positions, const float* q_gain,
+                                const float* k_gain, const float* inv_freq, int N, int Hq, int Hkv, int D,
+                                int rotary_dim, int BS, float eps, hipStream_t stream) {
+    const int heads = Hq + 2 * Hkv;
+    // few tokens: one head per wave; many tokens: a workgroup walks all heads of its token
+    const int hpw = N >= 256 ? (heads + 3) / 4 : 1;
+    const dim3 grid(N, (heads + 4 * hpw - 1) / (4 * hpw));
+#define SOC_QK_ARGS (const T*)qkv, (T*)q_out, (T*)k_out, (T*)v_out, (T*)k_pool, (T*)v_pool, block_table, \
+        table_width, token_rows, positions, q_gain, k_gain, inv_freq, Hq, Hkv, D, rotary_dim, BS, eps, hpw
+    if (D <= 64) hipLaunchKernelGGL((qk_norm_rope_kernel<T, 1>), grid, dim3(256), 0, stream, SOC_QK_ARGS);
+    else if (D <= 128) hipLaunchKernelGGL((qk_norm_rope_kernel<T, 2>), grid, dim3(256), 0, stream, SOC_QK_ARGS);
+    else hipLaunchKernelGGL((qk_norm_rope_kernel<T, 4>), grid, dim3(256), 0, stream, SOC_QK_ARGS);
+#undef SOC_QK_ARGS
 }
 
 SOC_EXPORT int soc_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void* v_out, void* k_pool,
@@ -298,20 +380,20 @@ SOC_EXPORT int soc_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void*
                                 int D, int rotary_dim, int BS, float eps, int dtype,
                                 hipStream_t stream) {
     if (N <= 0) return 0;
-    if (D > SOC_MAX_HEAD || D < 1) return (int)hipErrorInvalidValue;
-    const int head_groups = (Hq + 2 * Hkv + 3) / 4;
-    if (head_groups > 65535) return (int)hipErrorInvalidValue;
-    const dim3 grid(N, head_groups);
+    if (D > SOC_MAX_HEAD || D < 1 || D % 4) return (int)hipErrorInvalidValue;
+    if ((Hq + 2 * Hkv + 3) / 4 > 65535) return (int)hipErrorInvalidValue;
+    // a lane owns 1, 2 or 4 consecutive elements (head size up to 64, 128, 256); half the
+    // rotary width must be a whole number of lanes
+    const int ve = D <= 64 ? 1 : (D <= 128 ? 2 : 4);
+    if (inv_freq && (rotary_dim % (2 * ve) || rotary_dim > D)) return (int)hipErrorInvalidValue;
     if (dtype == 0)
-        hipLaunchKernelGGL(qk_norm_rope_kernel<float>, grid, dim3(256), 0, stream, (const float*)qkv,
-                           (float*)q_out, (float*)k_out, (float*)v_out, (float*)k_pool, (float*)v_pool,
-                           block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
-                           Hq, Hkv, D, rotary_dim, BS, eps);
+        launch_qk_norm_rope<float>(qkv, q_out, k_out, v_out, k_pool, v_pool, block_table, table_width,
+                                   token_rows, positions, q_gain, k_gain, inv_freq, N, Hq, Hkv, D,
+                                   rotary_dim, BS, eps, stream);
     else
-        hipLaunchKernelGGL(qk_norm_rope_kernel<bf16>, grid, dim3(256), 0, stream, (const bf16*)qkv,
-                           (bf16*)q_out, (bf16*)k_out, (bf16*)v_out, (bf16*)k_pool, (bf16*)v_pool,
-                           block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq,
-                           Hq, Hkv, D, rotary_dim, BS, eps);
+        launch_qk_norm_rope<bf16>(qkv, q_out, k_out, v_out, k_pool, v_pool, block_table, table_width,
+                                  token_rows, positions, q_gain, k_gain, inv_freq, N, Hq, Hkv, D,
+                                  rotary_dim, BS, eps, stream);
     return soc_last_error();
 }
 
