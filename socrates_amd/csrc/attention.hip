@@ -16,6 +16,7 @@
 // paged_attn_reduce_kernel merges the key splits of a token
 // (model/kernels/csrc/paged_attention.cu:278-297).
 #include "common.h"
+#include <type_traits>
 
 #ifndef SOC_HEAD_DIM
 #error "compile with -DSOC_HEAD_DIM=<head size>"
@@ -587,17 +588,27 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
 // =============================================================================================
 // Prompt portions (bfloat16): a workgroup of four waves owns 4 * RT * 16 rows of one sequence
 // and kv head (consecutive tokens x the heads of the group) and walks the keys 32 at a time.
-// The four waves load each K and V tile once, together, into LDS (V transposed on the way,
-// so that a slice of V^T for the second product is one 8-byte read), which cuts the traffic
-// from L2 by four against one wave per row block. Tiles are double-buffered in LDS and the
-// next tile's global loads are issued before the current tile's products. Products, softmax
-// and layouts are those of paged_attn_mfma_kernel; the second product takes 32 keys per MFMA.
+// The four waves load each K and V tile once, together, into LDS, which cuts the traffic from
+// L2 by four against one wave per row block. Tiles are double-buffered in LDS; the global
+// loads of the next tile are issued before the products of the current one, and the pages of
+// the tile after that are looked up at the same time, so no wave waits for a lookup.
+//
+// Layouts. A lane owns eight consecutive keys of a tile (8 * (lane / 16) ..): K rows are
+// stored in LDS in the order in which the two 16-key products want them (row 16 * sub + i
+// holds key 8 * (i / 4) + 4 * sub + i % 4), so that the scores of a lane, from both products,
+// are those eight keys, which is what the 32-key second product wants as operand B. V is
+// stored transposed ([d][key], two keys packed per word on the way in), so that a lane's
+// slice of V^T is 16 contiguous bytes. Softmax runs in base 2 (scores times scale * log2 e)
+// in float32. Tiles that every row of a wave sees whole take a path without masks.
 constexpr int PF_KEYS = 32;
 constexpr int PF_K_STRIDE = D + 8;                  // K tile [32][D + 8]
 constexpr int PF_V_STRIDE = PF_KEYS + 4;            // V^T tile [D][32 + 4]
-constexpr int PF_CHUNKS = PF_KEYS * D / 8;          // 16-byte chunks per tile and operand
-constexpr int PF_PER_THREAD = (PF_CHUNKS + 255) / 256;
 constexpr int PF_K_ELEMS = PF_KEYS * PF_K_STRIDE, PF_V_ELEMS = D * PF_V_STRIDE;
+constexpr int PF_PARTS = D / 8;                     // 16-byte chunks of one key
+
+__device__ __forceinline__ int pf_k_row(int k) {    // LDS row of key k of a tile
+    return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3);
+}
 
 template <int RT>
 __global__ void __launch_bounds__(256)
@@ -605,15 +616,17 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                           const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
                           int table_width, const int* __restrict__ token_rows,
                           const int* __restrict__ positions, const int* __restrict__ row_blocks,
-                          bf16* __restrict__ out, int Hq, int Hkv, int BS, float scale, int window,
-                          int group_pad_log2) {
+                          bf16* __restrict__ out, int Hq, int Hkv, int BS, int bs_shift, float scale,
+                          int window, int group_pad_log2) {
+    static_assert(D <= 128, "one key pair per thread");
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][PF_K_ELEMS];
     __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][PF_V_ELEMS];
     const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
     const int li = lane % 16, kb = lane / 16;
     const int G = Hq / Hkv, Gp = 1 << group_pad_log2;
     const int chunks = (G + 15) / 16;
-    const int blk = blockIdx.x / (Hkv * chunks);
+    // late row blocks see the most keys: they go first, so that the short ones fill the end
+    const int blk = (int)(gridDim.x / (Hkv * chunks)) - 1 - (int)(blockIdx.x / (Hkv * chunks));
     const int kvh = (blockIdx.x / chunks) % Hkv, chunk = blockIdx.x % chunks;
     const int tok0 = row_blocks[2 * blk], ntok = row_blocks[2 * blk + 1];
     const int pos0 = positions[tok0];
@@ -625,8 +638,10 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int klo = kmin & ~(PF_KEYS - 1);
     // this wave's rows
     const int wtok0 = wave * tokens_per_wave;                       // first token of the wave in the block
-    const int wave_hi = min(khi, pos0 + wtok0 + tokens_per_wave);   // keys past this are hidden from the wave
+    const int wave_lo_pos = pos0 + wtok0;                           // its first and last positions
+    const int wave_hi_pos = min(khi, wave_lo_pos + tokens_per_wave) - 1;
     const bool wave_has_rows = wtok0 < ntok;
+    const float c2 = scale * 1.44269504088896340736f;               // to base 2
 
     int row_pos[RT];
     size_t row_q[RT];
@@ -651,114 +666,182 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     }
 
-    // cooperative tile loads: thread -> chunks (key, part) of K and of V
-    uint4 kr[PF_PER_THREAD], vr[PF_PER_THREAD];
-    auto fetch = [&](int key0) {
+    // Cooperative tile loads: a thread owns two neighbouring keys (2 kp, 2 kp + 1) and one
+    // 16-byte part of them, of K and of V. Keys that no row of the block sees are never read;
+    // zeros stand in for them.
+    const int kp = tid % 16, part = tid / 16;
+    const bool loader = part < PF_PARTS;
+    const size_t page_stride = (size_t)Hkv * BS * D;
+    const bf16* k_base = k_pool + (size_t)kvh * BS * D + part * 8;
+    const bf16* v_base = v_pool + (size_t)kvh * BS * D + part * 8;
+    const bool pair_in_page = bs_shift >= 1;           // keys 2 kp and 2 kp + 1 share a page
+    // a tile inside [kmin, khi) needs no predicate
+    auto lookup = [&](int key0, int (&pg)[2]) {
+        if (!loader) { pg[0] = pg[1] = -1; return; }
+        if (pair_in_page && key0 >= kmin && key0 + PF_KEYS <= khi) {
+            pg[0] = pg[1] = table[(key0 + 2 * kp) >> bs_shift];
+            return;
+        }
 #pragma unroll
-        for (int j = 0; j < PF_PER_THREAD; ++j) {
-            const int c = tid + 256 * j;
-            const int ck = c / (D / 8), part = c % (D / 8);
-            const int key = key0 + ck;
-            if ((PF_CHUNKS % 256 == 0 || c < PF_CHUNKS) && key >= kmin && key < khi) {
-                const size_t off = ((size_t)table[key / BS] * Hkv * BS + (size_t)kvh * BS + key % BS) * D + part * 8;
-                kr[j] = *reinterpret_cast<const uint4*>(k_pool + off);
-                vr[j] = *reinterpret_cast<const uint4*>(v_pool + off);
+        for (int h = 0; h < 2; ++h) {
+            const int key = key0 + 2 * kp + h;
+            pg[h] = (key >= kmin && key < khi) ? table[bs_shift >= 0 ? key >> bs_shift : key / BS] : -1;
+        }
+    };
+    auto fetch = [&](int key0, const int (&pg)[2], uint4 (&kr)[2], uint4 (&vr)[2]) {
+        if (!loader) return;
+        if (pair_in_page && key0 >= kmin && key0 + PF_KEYS <= khi) {
+            const size_t off = (size_t)pg[0] * page_stride + (size_t)(((key0 + 2 * kp) & (BS - 1)) * D);
+            kr[0] = *reinterpret_cast<const uint4*>(k_base + off);
+            kr[1] = *reinterpret_cast<const uint4*>(k_base + off + D);
+            vr[0] = *reinterpret_cast<const uint4*>(v_base + off);
+            vr[1] = *reinterpret_cast<const uint4*>(v_base + off + D);
+            return;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int key = key0 + 2 * kp + h;
+            if (pg[h] >= 0) {
+                const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
+                const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
+                kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
+                vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
             } else {
-                kr[j] = make_uint4(0u, 0u, 0u, 0u);                  // unseen keys are never read
-                vr[j] = make_uint4(0u, 0u, 0u, 0u);
+                kr[h] = make_uint4(0u, 0u, 0u, 0u);
+                vr[h] = make_uint4(0u, 0u, 0u, 0u);
             }
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
+        if (!loader) return;
+        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp) * PF_K_STRIDE + part * 8]) = kr[0];
+        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp + 1) * PF_K_STRIDE + part * 8]) = kr[1];
+        const uint32_t a[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
+        const uint32_t b[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
+        uint32_t* vt = reinterpret_cast<uint32_t*>(&v_lds[buf][(part * 8) * PF_V_STRIDE + 2 * kp]);
 #pragma unroll
-        for (int j = 0; j < PF_PER_THREAD; ++j) {
-            const int c = tid + 256 * j;
-            if (PF_CHUNKS % 256 == 0 || c < PF_CHUNKS) {
-                const int ck = c / (D / 8), part = c % (D / 8);
-                *reinterpret_cast<uint4*>(&k_lds[buf][ck * PF_K_STRIDE + part * 8]) = kr[j];
-                const uint32_t w4[4] = {vr[j].x, vr[j].y, vr[j].z, vr[j].w};
-                uint16_t* vt = &v_lds[buf][(part * 8) * PF_V_STRIDE + ck];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    vt[(2 * e) * PF_V_STRIDE] = (uint16_t)(w4[e] & 0xffffu);
-                    vt[(2 * e + 1) * PF_V_STRIDE] = (uint16_t)(w4[e] >> 16);
-                }
-            }
+        for (int e = 0; e < 4; ++e) {
+            // element 2e and 2e+1 of both keys: (key 2kp in the low half, key 2kp+1 in the high)
+            vt[(2 * e) * (PF_V_STRIDE / 2)] = __builtin_amdgcn_perm(b[e], a[e], 0x05040100u);
+            vt[(2 * e + 1) * (PF_V_STRIDE / 2)] = __builtin_amdgcn_perm(b[e], a[e], 0x07060302u);
         }
     };
 
-    if (klo < khi) { fetch(klo); stash(0); }
-    __syncthreads();
-    int buf = 0;
-    for (int key0 = klo; key0 < khi; key0 += PF_KEYS) {
-        const bool more = key0 + PF_KEYS < khi;
-        if (more) fetch(key0 + PF_KEYS);
-        if (wave_has_rows && key0 < wave_hi) {
-            const uint16_t* kt = k_lds[buf];
-            const uint16_t* vt = v_lds[buf];
-            s16x4_t pf[RT][2];
-            float alpha[RT];
-            bool any_rescale = false;
+    // One tile for this wave's rows. MASKED: some key of the tile is hidden from some row.
+    auto compute = [&](int key0, int buf, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const uint16_t* kt = k_lds[buf];
+        const uint16_t* vt = v_lds[buf];
+        uint4 ka[QK_STEPS], kc[QK_STEPS];
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                f32x4_t s0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, s1 = s0;
-#pragma unroll
-                for (int kk = 0; kk < QK_STEPS; ++kk) {
-                    const uint4 ka = load_qk_slice(reinterpret_cast<const bf16*>(kt + li * PF_K_STRIDE), kk, kb);
-                    const uint4 kc = load_qk_slice(reinterpret_cast<const bf16*>(kt + (16 + li) * PF_K_STRIDE), kk, kb);
-                    s0 = qk_mfma(ka, qf[rt][kk], s0);
-                    s1 = qk_mfma(kc, qf[rt][kk], s1);
-                }
-                float sv[8];
-                float mx = -INFINITY;
-#pragma unroll
-                for (int r = 0; r < 8; ++r) {
-                    const int key = key0 + (r < 4 ? 0 : 16) + 4 * kb + (r & 3);
-                    bool seen = key <= row_pos[rt] && key < khi;
-                    if (window > 0) seen = seen && key > row_pos[rt] - window;
-                    sv[r] = seen ? (r < 4 ? s0[r & 3] : s1[r & 3]) * scale : -INFINITY;
-                    mx = fmaxf(mx, sv[r]);
-                }
-                mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
-                const float mn = fmaxf(m[rt], mx);
-                const float ms = mn == -INFINITY ? 0.f : mn;
-                alpha[rt] = __expf(m[rt] - ms);
-                float psum = 0.f;
-                uint16_t pb[8];
-#pragma unroll
-                for (int r = 0; r < 8; ++r) {
-                    const float p = __expf(sv[r] - ms);
-                    psum += p;
-                    pb[r] = f32_to_bf16_bits(p);
-                }
-                l[rt] = l[rt] * alpha[rt] + psum;
-                any_rescale = any_rescale || (m[rt] != mn);
-                m[rt] = mn;
-                pf[rt][0] = (s16x4_t){(short)pb[0], (short)pb[1], (short)pb[2], (short)pb[3]};
-                pf[rt][1] = (s16x4_t){(short)pb[4], (short)pb[5], (short)pb[6], (short)pb[7]};
-            }
-            if (__any(any_rescale)) {
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                    for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
-            }
-#pragma unroll
-            for (int j = 0; j < DV; ++j) {
-                const uint16_t* src = vt + (j * 16 + li) * PF_V_STRIDE + 4 * kb;
-                const s16x4_t va = *reinterpret_cast<const s16x4_t*>(src);          // keys 4kb .. 4kb+3
-                const s16x4_t vc = *reinterpret_cast<const s16x4_t*>(src + 16);     // keys 16+4kb ..
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                    o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pf[rt][0], o[rt][j], 0, 0, 0);
-                    o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vc, pf[rt][1], o[rt][j], 0, 0, 0);
-                }
-            }
+        for (int kk = 0; kk < QK_STEPS; ++kk) {
+            ka[kk] = load_qk_slice(reinterpret_cast<const bf16*>(kt + li * PF_K_STRIDE), kk, kb);
+            kc[kk] = load_qk_slice(reinterpret_cast<const bf16*>(kt + (16 + li) * PF_K_STRIDE), kk, kb);
         }
-        if (more) stash(buf ^ 1);           // the other buffer: nobody reads it in this iteration
+        uint4 pf[RT];
+        float alpha[RT];
+        bool any_rescale = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            f32x4_t s0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) {
+                s0 = qk_mfma(ka[kk], qf[rt][kk], s0);
+                s1 = qk_mfma(kc[kk], qf[rt][kk], s1);
+            }
+            float t[8];
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                t[r] = (r < 4 ? s0[r & 3] : s1[r & 3]) * c2;
+                if constexpr (MASKED) {
+                    const int key = key0 + 8 * kb + r;
+                    bool seen = key <= row_pos[rt];
+                    if (window > 0) seen = seen && key > row_pos[rt] - window;
+                    t[r] = seen ? t[r] : -INFINITY;
+                }
+                mx = fmaxf(mx, t[r]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
+            const float mn = fmaxf(m[rt], mx);
+            const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
+            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - ms);
+            float p[8];
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(t[r] - ms);
+                psum += p[r];
+            }
+            l[rt] = l[rt] * alpha[rt] + psum;
+            any_rescale = any_rescale || (m[rt] != mn);
+            m[rt] = mn;
+            pf[rt] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
+                                pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
+        }
+        if (__any(any_rescale)) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
+        }
+        // O^T += V^T P^T over the 32 keys, one 16-wide block of d at a time
+        uint4 va[DV];
+#pragma unroll
+        for (int j = 0; j < DV; ++j) {
+            const uint2* src = reinterpret_cast<const uint2*>(vt + (j * 16 + li) * PF_V_STRIDE + 8 * kb);
+            const uint2 lo = src[0], hi = src[1];
+            va[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+#pragma unroll
+        for (int j = 0; j < DV; ++j)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                o[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    *reinterpret_cast<const bf16x8_t*>(&va[j]), *reinterpret_cast<const bf16x8_t*>(&pf[rt]),
+                    o[rt][j], 0, 0, 0);
+    };
+
+    // Two tiles of global loads are in flight while one is computed: at the top of the
+    // iteration of tile t, tile t sits in LDS buffer t % 2, the loads of tile t + 1 are on
+    // their way into one pair of staging registers, and the pages of tile t + 2 were asked
+    // for. The iteration issues the lookup of tile t + 3 and the loads of tile t + 2, computes,
+    // and then moves tile t + 1 from its registers to the other LDS buffer, which nobody has
+    // read since the barrier that ended the previous iteration.
+    auto tile = [&](int key0, int buf) {
+        if (wave_has_rows && key0 <= wave_hi_pos) {
+            // whole: every key of the tile is at or before the wave's first position and inside
+            // the window of its last one
+            const bool whole = key0 + PF_KEYS - 1 <= wave_lo_pos &&
+                               (window <= 0 || key0 > wave_hi_pos - window);
+            if (whole) compute(key0, buf, std::false_type{});
+            else compute(key0, buf, std::true_type{});
+        }
+    };
+    // Loads return in order, so a lookup is issued before the tile loads of its iteration:
+    // waiting for it then leaves those tile loads in flight.
+    int pg0[2], pg1[2];
+    uint4 kr0[2], vr0[2], kr1[2], vr1[2];
+    lookup(klo, pg0);
+    lookup(klo + PF_KEYS, pg1);
+    fetch(klo, pg0, kr0, vr0);
+    lookup(klo + 2 * PF_KEYS, pg0);
+    fetch(klo + PF_KEYS, pg1, kr1, vr1);
+    stash(0, kr0, vr0);
+    __syncthreads();
+    for (int key0 = klo; key0 < khi; key0 += 2 * PF_KEYS) {
+        lookup(key0 + 3 * PF_KEYS, pg1);
+        fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
+        tile(key0, 0);
+        stash(1, kr1, vr1);
         __syncthreads();
-        buf ^= 1;
+        if (key0 + PF_KEYS >= khi) break;
+        lookup(key0 + 4 * PF_KEYS, pg0);
+        fetch(key0 + 3 * PF_KEYS, pg1, kr1, vr1);
+        tile(key0 + PF_KEYS, 1);
+        stash(0, kr0, vr0);
+        __syncthreads();
     }
 
 #pragma unroll
@@ -771,15 +854,16 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 #pragma unroll
         for (int j = 0; j < DV; ++j) {
             uint2 pk;
-            pk.x = (uint32_t)f32_to_bf16_bits(o[rt][j][0] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][1] * inv) << 16);
-            pk.y = (uint32_t)f32_to_bf16_bits(o[rt][j][2] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][3] * inv) << 16);
+            pk.x = pack_bf16x2(o[rt][j][0] * inv, o[rt][j][1] * inv);
+            pk.y = pack_bf16x2(o[rt][j][2] * inv, o[rt][j][3] * inv);
             *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
         }
     }
 }
 
-// bfloat16 only, no key splits. row_blocks [n_row_blocks, 2] = (first token, tokens) of each
-// block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of one sequence.
+// bfloat16 only, head sizes up to 128, no key splits. row_blocks [n_row_blocks, 2] = (first
+// token, tokens) of each block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of
+// one sequence.
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
@@ -792,16 +876,23 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
     const long groups = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     if (groups > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    int bs_shift = -1;
+    if ((BS & (BS - 1)) == 0)
+        for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
+    if constexpr (D <= 128) {
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
-        token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, scale, window, group_pad_log2
-    if (row_tiles == 1)
-        hipLaunchKernelGGL(paged_attn_prefill_kernel<1>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-    else if (row_tiles == 2)
-        hipLaunchKernelGGL(paged_attn_prefill_kernel<2>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-    else
-        return (int)hipErrorInvalidValue;
+        token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2
+        if (row_tiles == 1)
+            hipLaunchKernelGGL(paged_attn_prefill_kernel<1>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+        else if (row_tiles == 2)
+            hipLaunchKernelGGL(paged_attn_prefill_kernel<2>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+        else
+            return (int)hipErrorInvalidValue;
 #undef SOC_PF_ARGS
-    return soc_last_error();
+        return soc_last_error();
+    } else {
+        return (int)hipErrorInvalidValue;
+    }
 }
 
 SOC_EXPORT int soc_attention_head_dim() { return D; }

@@ -16,11 +16,17 @@ struct bf16 { uint16_t bits; };
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16 v) { return __uint_as_float(((uint32_t)v.bits) << 16); }
 
+// Round to nearest even; gfx950 converts in hardware (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);   // quiet NaN
-    u += 0x7fffu + ((u >> 16) & 1u);                                                // nearest even
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+// Two floats to two bfloat16 in one word, `lo` in the low half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    typedef float soc_f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 soc_bf16x2 __attribute__((ext_vector_type(2)));
+    const soc_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, soc_bf16x2));
 }
 
 template <typename T> __device__ __forceinline__ T from_float(float v);

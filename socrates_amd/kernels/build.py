@@ -33,6 +33,11 @@ ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-fno-gpu-rdc", "-Wno-unused-value"]
+# Attention up to head size 128: MFMA accumulators stay in ordinary vector registers. The
+# softmax rescales them with vector instructions, and copies to and from the accumulation
+# registers would cost more than the products. Larger heads need both register files.
+MFMA_VGPR_FLAGS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+MFMA_VGPR_MAX_HEAD = 128
 
 SOURCES = {"elementwise": "elementwise.hip", "gemm": "gemm.hip", "sampling": "sampling.hip",
            "attention": "attention.hip"}
@@ -80,7 +85,8 @@ def _variant(name: str, head_dim=None):
     if name == "attention":
         if head_dim is None:
             raise ValueError("the attention library is built per head size")
-        return f"attention_d{head_dim}", [f"-DSOC_HEAD_DIM={head_dim}"]
+        extra = MFMA_VGPR_FLAGS if head_dim <= MFMA_VGPR_MAX_HEAD else []
+        return f"attention_d{head_dim}", [f"-DSOC_HEAD_DIM={head_dim}"] + extra
     return name, []
 
 
