@@ -219,7 +219,8 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
                         int k_per_wave) {
     __shared__ float red[SK_MAX_WAVES * MT * RW * 256];
-    const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
+    // the wave index is the same in all lanes: say so, and the K loop runs on scalar registers
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
     const int n0 = blockIdx.x * 16 * RW;
     const int li = lane % 16, lk = (lane / 16) * 8;
@@ -236,28 +237,31 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
         w_ok[r] = n0 + r * 16 + li < N;
         w_off[r] = (size_t)(w_ok[r] ? n0 + r * 16 + li : 0) * K + lk;
     }
-    size_t x_off[MT];
-    bool x_ok[MT];
+    // X is read through a buffer descriptor that covers its M rows: a lane whose row lies
+    // outside (M = 8 leaves half of the 16 lanes of a tile without one) gets zeros and asks
+    // memory for nothing. X comes from L2 for every workgroup, so this halves that traffic.
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, M * K * 2, 0x00020000);
+    uint32_t x_off[MT];                                  // bytes
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        x_ok[t] = t * 16 + li < M;
-        x_off[t] = (size_t)(x_ok[t] ? t * 16 + li : 0) * K + lk;
-    }
+    for (int t = 0; t < MT; ++t) x_off[t] = (uint32_t)(((t * 16 + li) * K + lk) * 2);
     f32x4 acc[MT][RW];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int r = 0; r < RW; ++r) acc[t][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    // Full steps of 128 k load without any predicate (a row outside the matrix reads row 0
-    // and its results are dropped at the store), so the loop body is straight-line code and
-    // the loads of the next step stay in flight under the MFMAs of the current one.
+    // Full steps of 128 k load without any predicate (a weight row outside the matrix reads
+    // row 0 and its results are dropped at the store; X rows outside read zeros through the
+    // descriptor), so the loop body is straight-line code and the loads of the next step stay
+    // in flight under the MFMAs of the current one.
 #define SK_LOAD(B, K0)                                                                              \
     _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u) {                                          \
         _Pragma("unroll") for (int r = 0; r < RW; ++r)                                               \
             B.w[r][u] = *reinterpret_cast<const uint4*>(W + w_off[r] + (K0) + 32 * u);               \
         _Pragma("unroll") for (int t = 0; t < MT; ++t)                                               \
-            B.x[t][u] = *reinterpret_cast<const uint4*>(X + x_off[t] + (K0) + 32 * u);               \
+            B.x[t][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(              \
+                x_rsrc, x_off[t] + (uint32_t)(((K0) + 32 * u) * 2), 0, 0));                          \
     }
 #define SK_COMPUTE(B)                                                                               \
     _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u)                                            \
@@ -301,7 +305,9 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
                 b0.w[r][u] = in ? *reinterpret_cast<const uint4*>(W + w_off[r] + kk) : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
             for (int t = 0; t < MT; ++t)
-                b0.x[t][u] = in ? *reinterpret_cast<const uint4*>(X + x_off[t] + kk) : make_uint4(0u, 0u, 0u, 0u);
+                b0.x[t][u] = in ? __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                      x_rsrc, x_off[t] + (uint32_t)(kk * 2), 0, 0))
+                                : make_uint4(0u, 0u, 0u, 0u);
         }
         SK_COMPUTE(b0)
     }
@@ -359,7 +365,7 @@ static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, in
 SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C, int M, int N, int K,
                                            int c_dtype, int n_waves, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K % 8 || K < 8 || N % 32) return (int)hipErrorInvalidValue;
+    if (M > 16 || K % 8 || K < 8 || K > (1 << 23) || N % 32) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > SK_MAX_WAVES) return (int)hipErrorInvalidValue;
     const int k_per_wave = ((K + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
     const int k_per_split = k_per_wave * n_waves;
@@ -400,7 +406,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
                                     int K, int c_dtype, int row_tiles, int n_waves, int k_splits,
                                     hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 64 || K % 8 || K < 8) return (int)hipErrorInvalidValue;
+    if (M > 64 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;   // 32-bit byte offsets into X
     if (n_waves < 1 || n_waves > SK_MAX_WAVES || k_splits < 1 || k_splits > 65535)
         return (int)hipErrorInvalidValue;
     if ((k_splits > 1) != (Cpart != nullptr)) return (int)hipErrorInvalidValue;

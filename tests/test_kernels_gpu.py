@@ -253,21 +253,25 @@ def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     hip.attention_workgroup = True
 
 
-@pytest.mark.parametrize("Hq,Hkv,D,bs", [(4, 2, 16, 16), (9, 3, 48, 4), (32, 8, 128, 16), (16, 1, 64, 32), (40, 2, 32, 8)])
+@pytest.mark.parametrize("Hq,Hkv,D,bs", [(4, 2, 16, 16), (9, 3, 48, 4), (32, 8, 128, 16), (16, 1, 64, 32), (40, 2, 32, 8),
+                                         (8, 2, 64, 12), (4, 4, 32, 1), (6, 2, 128, 24), (3, 1, 112, 2)])
 def test_prefill_attention_whole_prompts(kernel_sets, Hq, Hkv, D, bs):
     """Whole prompts and long portions through the workgroup kernel: several sequences of
-    uneven length, one of them continuing a cache of 100 tokens."""
+    uneven length, one of them continuing a cache of 100 tokens; page sizes that are powers of
+    two (two neighbouring keys share a page), one, and no power of two; with and without a
+    window (tiles that lie partly or wholly before the window's start)."""
     hip, _ = kernel_sets[torch.bfloat16]
     lens = [257, 33, 100 + 75, 16]
     slot, dense = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=D + 1)
     rows = [0] * 257 + [1] * 33 + [2] * 75 + [3] * 16
     pos = list(range(257)) + list(range(33)) + list(range(100, 175)) + list(range(16))
     q = rnd((len(rows), Hq, D), torch.bfloat16, 21)
-    want = dense_attention(q, dense, rows, pos, D ** -0.5)
-    for rt in (1, 2):
-        hip.attention_row_tiles = rt
-        got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5)
-        close(got.cpu(), want, torch.bfloat16)
+    for window in (None, 40, 97):
+        want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
+        for rt in (1, 2):
+            hip.attention_row_tiles = rt
+            got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
+            close(got.cpu(), want, torch.bfloat16)
     hip.attention_row_tiles = None
 
 

@@ -296,3 +296,134 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(kind, dtype):
     x = plain.block(x, w, 2, cfg2, torch.arange(21))
     want = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
     torch.testing.assert_close(whole, want, **tol)
+
+
+# ---- a toy feed-forward with routing and a toy position encoding, registered from outside ------
+@dataclass(frozen=True)
+class RoutedSpec:
+    """y = p_e * Down_e(relu(Up_e x)) for the expert e with the largest router logit, p its
+    softmax probability."""
+    hidden: int
+    intermediate: int
+    n_experts: int
+
+
+class RoutedFeedForward:
+    @staticmethod
+    def tensors(spec):
+        t = {"router.weight": TensorDecl((spec.n_experts, spec.hidden), "vector")}
+        for e in range(spec.n_experts):
+            t[f"experts.{e}.up.weight"] = TensorDecl((spec.intermediate, spec.hidden))
+            t[f"experts.{e}.down.weight"] = TensorDecl((spec.hidden, spec.intermediate))
+        return t
+
+    def __init__(self, spec, tensors, ops):
+        self.spec, self.ops, self.t = spec, ops, tensors
+
+    def forward(self, x, ctx=None):
+        logits = x.float() @ self.t["router.weight"].float().T            # router in float32
+        prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        y = torch.zeros((x.shape[0], self.spec.hidden), dtype=torch.float32, device=x.device)
+        for e in range(self.spec.n_experts):
+            idx = (choice == e).nonzero().flatten()
+            if idx.numel() == 0:
+                continue
+            h = torch.relu(self.ops.linear(x[idx].contiguous(), self.t[f"experts.{e}.up.weight"]))
+            y[idx] = self.ops.linear(h, self.t[f"experts.{e}.down.weight"]).float() * prob[idx, None]
+        return y.to(self.ops.dtype)
+
+
+@dataclass(frozen=True)
+class PairRotationSpec:
+    """Rotation of neighbouring pairs (2i, 2i + 1) by position * theta^(-2i / head_dim): no
+    fused form is offered, so the attention part takes norm, apply and store as three steps."""
+    head_dim: int
+    theta: float
+
+
+class PairRotation:
+    @staticmethod
+    def tensors(spec):
+        return {}
+
+    def __init__(self, spec, tensors, ops):
+        self.spec = spec
+
+    def angles(self, positions):
+        D = self.spec.head_dim
+        inv = self.spec.theta ** (-torch.arange(0, D, 2, dtype=torch.float32, device=positions.device) / D)
+        a = positions.float()[:, None] * inv
+        return torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+
+    def rotate(self, x, cos, sin):
+        a, b = x[..., 0::2].float(), x[..., 1::2].float()
+        out = torch.stack([a * cos - b * sin, a * sin + b * cos], dim=-1).flatten(-2)
+        return out.to(x.dtype)
+
+    def apply(self, q, k, positions):
+        cos, sin = self.angles(positions)
+        q.copy_(self.rotate(q, cos, sin))
+        if k is not None and k.numel():
+            k.copy_(self.rotate(k, cos, sin))
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_a_toy_routed_feed_forward_and_a_toy_position_encoding(kind, dtype):
+    """Both are defined and registered here. The plan gives layer 0 the toy encoding and the
+    routed feed-forward and layer 1 the usual parts: one model, different parts per layer."""
+    register_part(RoutedSpec, RoutedFeedForward)
+    register_part(PairRotationSpec, PairRotation)
+    ops = kernels(kind, dtype)
+    hidden, D, E, ff, T = 32, 16, 3, 24, 21
+    att = AttentionSpec(hidden, 4, 2, D, D ** -0.5, RMSNormSpec(D, 1e-6), PairRotationSpec(D, 100.0))
+    toy = BlockSpec(att, RoutedSpec(hidden, ff, E), RMSNormSpec(hidden, 1e-6), RMSNormSpec(hidden, 1e-6),
+                    prefix="model.layers.0.")
+    plan = plan_with([toy, qwen_like_block(1)], [RunStep(0, 0), RunStep(1, 1)], hidden)
+    assert "model.layers.0.mlp.experts.2.down.weight" in expected_tensors(plan)
+    weights = random_tensors(expected_tensors(plan), seed=11, dtype=ops.dtype, device=ops.device, std=0.2, gain_std=0.1)
+    g = torch.Generator().manual_seed(12)
+    weights["model.layers.0.mlp.router.weight"] = torch.randn(E, hidden, generator=g).to(ops.device)
+    tokens = random_prompts([T], 50, seed=8)[0]
+    outs = []
+    for cut in ([T], [4, 1, 1, 8, 2, 5], [T - 1, 1]):
+        model = DecoderModel(plan, weights, ops)
+        cache = CacheManager(cache_needs(plan), 2, 64, 8, 16, ops.dtype, ops.device)
+        runner = ModelRunner(model, cache)
+        row = cache.open_row()
+        logits, t = [], 0
+        for n in cut:
+            logits.append(runner.step([StepEntry(row, tokens[t:t + n], list(range(n)))]).float().cpu())
+            t += n
+        outs.append(torch.cat(logits))
+    tol = dict(atol=2e-4, rtol=2e-4) if dtype == torch.float32 else dict(atol=0.2, rtol=5e-2)
+    torch.testing.assert_close(outs[1], outs[0], **tol)
+    torch.testing.assert_close(outs[2], outs[0], **tol)
+
+    # the same model from plain formulas
+    w = {n: t.float().cpu() for n, t in weights.items()}
+    pos = torch.arange(T)
+    x = w["embed.weight"][torch.tensor(tokens)]
+    p = "model.layers.0."
+    h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6)
+    inv = 100.0 ** (-torch.arange(0, D, 2).float() / D)
+    ang = pos.float()[:, None] * inv
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+    def pairs(t):
+        a, b = t[..., 0::2], t[..., 1::2]
+        return torch.stack([a * cos - b * sin, a * sin + b * cos], dim=-1).flatten(-2)
+
+    q = pairs(plain.rms_norm((h @ w[p + "self_attn.q_proj.weight"].T).view(T, 4, D), w[p + "self_attn.q_norm.weight"], 1e-6))
+    k = pairs(plain.rms_norm((h @ w[p + "self_attn.k_proj.weight"].T).view(T, 2, D), w[p + "self_attn.k_norm.weight"], 1e-6))
+    v = (h @ w[p + "self_attn.v_proj.weight"].T).view(T, 2, D)
+    x = x + plain.attention_scores(q, k, v, D ** -0.5).reshape(T, 4 * D) @ w[p + "self_attn.o_proj.weight"].T
+    h = plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6)
+    prob, choice = torch.softmax(h @ w[p + "mlp.router.weight"].T, dim=-1).max(dim=-1)
+    y = torch.stack([prob[t] * (torch.relu(h[t] @ w[p + f"mlp.experts.{int(choice[t])}.up.weight"].T)
+                                @ w[p + f"mlp.experts.{int(choice[t])}.down.weight"].T) for t in range(T)])
+    assert len(set(choice.tolist())) > 1                       # the router does choose
+    x = x + y
+    cfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6, rope_theta=1e4)
+    x = plain.block(x, w, 1, cfg, pos)
+    want = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
+    torch.testing.assert_close(outs[0], want, **tol)
