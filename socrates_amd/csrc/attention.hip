@@ -506,24 +506,76 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             }
         } else {
             const size_t pi = (base / D) * n_splits + split;
+            if (m[rt] != -INFINITY) {                        // the merge reads nothing of an empty split
 #pragma unroll
-            for (int j = 0; j < DV; ++j)
-                *reinterpret_cast<float4*>(part_o + pi * D + j * 16 + 4 * kb) =
-                    make_float4(o[rt][j][0], o[rt][j][1], o[rt][j][2], o[rt][j][3]);
+                for (int j = 0; j < DV; ++j)
+                    *reinterpret_cast<float4*>(part_o + pi * D + j * 16 + 4 * kb) =
+                        make_float4(o[rt][j][0], o[rt][j][1], o[rt][j][2], o[rt][j][3]);
+            }
             if (kb == 0) { part_ml[pi * 2] = m[rt]; part_ml[pi * 2 + 1] = L; }
         }
     }
 }
 
-// Merge all n_splits partials of a (token, head); an empty split has m = -inf. One wave per
-// (token, head): first the splits lie across the lanes (maximum, weights, sum), then the head
-// dimension does, each lane adding its elements over the splits in order.
+// Merge all n_splits partials of a (token, head); an empty split has m = -inf and is not
+// read. One wave per (token, head): first the splits lie across the lanes (maximum, weights,
+// sum); then a lane owns four elements of the head dimension and every D / 4 lanes form a
+// group that adds every (64 / (D / 4))-th split, in order; the groups are added in order.
 __global__ void __launch_bounds__(64)
 paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                         bf16* __restrict__ out, int Hq, int n_splits) {
+    constexpr int LPG = D / 4;                              // lanes of a group
+    constexpr int NG = SOC_WAVE / LPG;                      // groups of a wave
     __shared__ float weight[256];
+    __shared__ __attribute__((aligned(16))) float4 red[SOC_WAVE];
     const int h = blockIdx.x, n = blockIdx.y, lane = threadIdx.x;
     const size_t base = ((size_t)n * Hq + h) * n_splits;
+    constexpr int FAST = 16;                                // partials a lane holds on the short path
+    if (n_splits <= SOC_WAVE && n_splits <= FAST * NG) {
+        // Few splits: every load is issued before any is needed (one trip to memory instead
+        // of two). An empty split's partial was never written: it is loaded, but not used.
+        const int sg = lane / LPG, e4 = lane % LPG;
+        const float ms = lane < n_splits ? part_ml[(base + lane) * 2] : -INFINITY;
+        const float ls = lane < n_splits ? part_ml[(base + lane) * 2 + 1] : 0.f;
+        float4 v[FAST];
+#pragma unroll
+        for (int j = 0; j < FAST; ++j) {
+            const int s = sg + j * NG;
+            v[j] = (sg < NG && s < n_splits)
+                       ? *reinterpret_cast<const float4*>(part_o + (base + s) * D + e4 * 4)
+                       : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        const float M = wave_max(ms);
+        const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+        const float L = wave_sum(w * ls);
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < FAST; ++j) {
+            const int s = sg + j * NG;
+            const float wj = __shfl(w, s < SOC_WAVE ? s : 0, SOC_WAVE);
+            if (sg < NG && s < n_splits && wj != 0.f) {
+                acc.x += v[j].x * wj; acc.y += v[j].y * wj; acc.z += v[j].z * wj; acc.w += v[j].w * wj;
+            }
+        }
+        if constexpr (NG > 1) {
+            red[lane] = acc;
+            __syncthreads();
+            if (lane < LPG) {
+                for (int g = 1; g < NG; ++g) {
+                    const float4 t = red[g * LPG + lane];
+                    acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+                }
+            }
+        }
+        if (lane < LPG) {
+            uint2 pk;
+            pk.x = pack_bf16x2(acc.x * inv, acc.y * inv);
+            pk.y = pack_bf16x2(acc.z * inv, acc.w * inv);
+            *reinterpret_cast<uint2*>(out + ((size_t)n * Hq + h) * D + e4 * 4) = pk;
+        }
+        return;
+    }
     float M = -INFINITY;
     for (int s = lane; s < n_splits; s += SOC_WAVE) M = fmaxf(M, part_ml[(base + s) * 2]);
     M = wave_max(M);
@@ -537,11 +589,31 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
     const float L = wave_sum(lsum);
     __syncthreads();
     const float inv = L > 0.f ? 1.0f / L : 0.f;
-    for (int e = lane; e < D; e += SOC_WAVE) {
-        float A = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < n_splits; ++s) A += part_o[(base + s) * D + e] * weight[s];
-        out[((size_t)n * Hq + h) * D + e] = from_float<bf16>(A * inv);
+    const int sg = lane / LPG, e4 = lane % LPG;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (sg < NG) {
+        for (int s = sg; s < n_splits; s += NG) {
+            const float w = weight[s];
+            if (w == 0.f) continue;
+            const float4 v = *reinterpret_cast<const float4*>(part_o + (base + s) * D + e4 * 4);
+            acc.x += v.x * w; acc.y += v.y * w; acc.z += v.z * w; acc.w += v.w * w;
+        }
+    }
+    if constexpr (NG > 1) {
+        red[lane] = acc;
+        __syncthreads();
+        if (lane < LPG) {
+            for (int g = 1; g < NG; ++g) {
+                const float4 v = red[g * LPG + lane];
+                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+            }
+        }
+    }
+    if (lane < LPG) {
+        uint2 pk;
+        pk.x = pack_bf16x2(acc.x * inv, acc.y * inv);
+        pk.y = pack_bf16x2(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2*>(out + ((size_t)n * Hq + h) * D + e4 * 4) = pk;
     }
 }
 

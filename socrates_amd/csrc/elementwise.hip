@@ -107,13 +107,80 @@ __global__ void add_rmsnorm_regs_kernel(float* __restrict__ residual, const T* _
     }
 }
 
+// The same with eight consecutive elements per thread and 16-byte accesses, for rows of a
+// multiple of eight elements up to 8 * 1024: fewer, wider loads, all issued before the first
+// is needed. blockDim = d / 8 rounded up to whole waves.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+add_rmsnorm_vec8_kernel(float* __restrict__ residual, const T* __restrict__ delta,
+                        const float* __restrict__ partials, int n_partials, size_t partial_stride,
+                        const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
+                        int d, float eps) {
+    __shared__ float scratch[16];
+    const int i = blockIdx.x;
+    const int n = rows ? rows[i] : i;
+    const int j = threadIdx.x * 8;
+    const bool in = j < d;
+    float v[8], g[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = g[e] = 0.f;
+    if (in) {
+        float* r = residual + (size_t)n * d + j;
+        VecLoad<float, 8>::load(r, v);
+        VecLoad<float, 8>::load(w + j, g);
+        if (delta) {
+            float t[8];
+            VecLoad<T, 8>::load(delta + (size_t)n * d + j, t);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += t[e];
+        }
+        if (partials) {
+            const float* dp = partials + (size_t)n * d + j;
+            for (int s = 0; s < n_partials; ++s) {
+                float t[8];
+                VecLoad<float, 8>::load(dp + s * partial_stride, t);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += t[e];
+            }
+        }
+        if (!rows && (delta || partials)) {
+            *reinterpret_cast<float4*>(r) = make_float4(v[0], v[1], v[2], v[3]);
+            *reinterpret_cast<float4*>(r + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    if (!in) return;
+    T* o = out + (size_t)i * d + j;
+    if constexpr (sizeof(T) == 2) {
+        uint4 pk;
+        pk.x = pack_bf16x2(v[0] * inv * g[0], v[1] * inv * g[1]);
+        pk.y = pack_bf16x2(v[2] * inv * g[2], v[3] * inv * g[3]);
+        pk.z = pack_bf16x2(v[4] * inv * g[4], v[5] * inv * g[5]);
+        pk.w = pack_bf16x2(v[6] * inv * g[6], v[7] * inv * g[7]);
+        *reinterpret_cast<uint4*>(o) = pk;
+    } else {
+        float* of = reinterpret_cast<float*>(o);
+        *reinterpret_cast<float4*>(of) = make_float4(v[0] * inv * g[0], v[1] * inv * g[1], v[2] * inv * g[2], v[3] * inv * g[3]);
+        *reinterpret_cast<float4*>(of + 4) = make_float4(v[4] * inv * g[4], v[5] * inv * g[5], v[6] * inv * g[6], v[7] * inv * g[7]);
+    }
+}
+
 template <typename T>
 static void launch_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
                                size_t partial_stride, const float* w, void* out, const int* rows, int n_out,
                                int d, float eps, hipStream_t stream) {
     constexpr int VPT = 8;
     const int threads = d <= 1024 ? 128 : (d <= 2048 ? 256 : (d <= 4096 ? 512 : 1024));
-    if (d <= VPT * threads)
+    const bool aligned = d % 8 == 0 && partial_stride % 4 == 0 &&
+                         ((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)partials | (uintptr_t)w | (uintptr_t)out) % 16 == 0;
+    if (aligned && d <= 8 * 1024)
+        hipLaunchKernelGGL(add_rmsnorm_vec8_kernel<T>, dim3(n_out), dim3((d / 8 + 63) / 64 * 64), 0, stream, residual,
+                           (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
+    else if (d <= VPT * threads)
         hipLaunchKernelGGL((add_rmsnorm_regs_kernel<T, VPT>), dim3(n_out), dim3(threads), 0, stream, residual,
                            (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
     else
