@@ -325,7 +325,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     const int blk = task / (Hkv * chunks);
     const int kvh = (task / chunks) % Hkv, chunk = task % chunks;
     const int split = blockIdx.y;
-    const int tok0 = row_blocks[2 * blk], ntok = row_blocks[2 * blk + 1];
+    // no list of row blocks: every token alone (a decode step), one dependent load fewer
+    const int tok0 = row_blocks ? row_blocks[2 * blk] : blk, ntok = row_blocks ? row_blocks[2 * blk + 1] : 1;
     const int pos0 = positions[tok0];
     const int* table = block_table + (size_t)token_rows[tok0] * table_width;
 
@@ -618,7 +619,8 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
 }
 
 // bfloat16 only. row_blocks [n_row_blocks, 2] = (first token, tokens) of each block of at most
-// (16 * row_tiles) >> group_pad_log2 tokens of one sequence; 2^group_pad_log2 >= min(G, 16).
+// (16 * row_tiles) >> group_pad_log2 tokens of one sequence, or null: every token is a block
+// of its own (n_row_blocks = N); 2^group_pad_log2 >= min(G, 16).
 // Splits are over absolute key indices: split s covers keys [s * split_len, (s + 1) * split_len),
 // split_len a multiple of 16; n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml
 // [N, Hq, n_splits, 2], which are written for every (row, split), empty ones with m = -inf.
@@ -631,6 +633,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
         return (int)hipErrorInvalidValue;
+    if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
@@ -700,7 +703,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // late row blocks see the most keys: they go first, so that the short ones fill the end
     const int blk = (int)(gridDim.x / (Hkv * chunks)) - 1 - (int)(blockIdx.x / (Hkv * chunks));
     const int kvh = (blockIdx.x / chunks) % Hkv, chunk = blockIdx.x % chunks;
-    const int tok0 = row_blocks[2 * blk], ntok = row_blocks[2 * blk + 1];
+    const int tok0 = row_blocks ? row_blocks[2 * blk] : blk, ntok = row_blocks ? row_blocks[2 * blk + 1] : 1;
     const int pos0 = positions[tok0];
     const int* table = block_table + (size_t)token_rows[tok0] * table_width;
     const int tokens_per_wave = (16 * RT) >> group_pad_log2;
@@ -935,7 +938,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 
 // bfloat16 only, head sizes up to 128, no key splits. row_blocks [n_row_blocks, 2] = (first
 // token, tokens) of each block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of
-// one sequence.
+// one sequence, or null: every token is a block of its own.
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
@@ -944,6 +947,7 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
                                            hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1) return (int)hipErrorInvalidValue;
+    if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
     const long groups = (long)n_row_blocks * Hkv * ((G + 15) / 16);

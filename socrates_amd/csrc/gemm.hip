@@ -207,26 +207,30 @@ SOC_EXPORT int soc_gemm_bf16_mfma(const void* A, const void* W, void* C, int M, 
 constexpr int SK_UNROLL = 4;            // 16-byte slices per lane, row and buffer (4 x 32 = 128 k)
 constexpr int SK_STEP = 32 * SK_UNROLL;
 constexpr int SK_MAX_WAVES = 8;
+constexpr int SK_MAX_WAVES_SWIGLU = 16;     // gate waves and up waves
 
 template <int MT, int RW> struct SkBuf { uint4 w[RW][SK_UNROLL]; uint4 x[MT][SK_UNROLL]; };
 
-// SWIGLU: the two row tiles of a workgroup are 16 gate rows and the 16 up rows of the same
-// output columns (the weight's rows are interleaved in blocks of 16); the epilogue writes
-// silu(gate) * up, [M, N / 2], instead of both products.
+// SWIGLU (RW = 1): the weight's rows are interleaved in blocks of 16, 16 gate rows and then
+// the 16 up rows of the same output columns. The first half of a workgroup's waves takes the
+// gate tile and the second half the up tile, each half splitting K; the epilogue writes
+// silu(gate) * up, [M, N / 2], instead of both products. (One tile per wave streams the
+// weights faster than two.)
 template <typename TC, int MT, int RW, bool SWIGLU = false>
-__global__ void __launch_bounds__(64 * SK_MAX_WAVES)
+__global__ void __launch_bounds__(64 * (SWIGLU ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES))
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
                         int k_per_wave) {
-    __shared__ float red[SK_MAX_WAVES * MT * RW * 256];
+    __shared__ float red[(SWIGLU ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES) * MT * RW * 256];
     // the wave index is the same in all lanes: say so, and the K loop runs on scalar registers
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
-    const int n0 = blockIdx.x * 16 * RW;
+    const int k_waves = SWIGLU ? n_waves / 2 : n_waves;        // waves that share one tile's K
+    const int n0 = SWIGLU ? blockIdx.x * 32 + (wave / k_waves) * 16 : blockIdx.x * 16 * RW;
     const int li = lane % 16, lk = (lane / 16) * 8;
     const int split_begin = blockIdx.y * k_per_split;
     const int split_end = min(K, split_begin + k_per_split);
-    const int k_begin = split_begin + wave * k_per_wave;
+    const int k_begin = split_begin + (wave % k_waves) * k_per_wave;
     const int k_end = min(split_end, k_begin + k_per_wave);
     // Element offsets of this lane's rows (offsets, not pointers: the loads stay global
     // loads); a row outside the matrix is never loaded.
@@ -322,15 +326,15 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
                 red[(((wave * MT + t) * RW + r) * 64 + lane) * 4 + e] = acc[t][r][e];
     __syncthreads();
     if constexpr (SWIGLU) {
-        static_assert(!SWIGLU || RW == 2, "gate and up tiles");
-        for (int idx = tid; idx < MT * 256; idx += blockDim.x) {
-            const int t = idx / 256, ln = (idx % 256) / 4, e = idx % 4;
+        static_assert(!SWIGLU || (RW == 1 && MT == 1), "one tile per wave, gate waves then up waves");
+        for (int idx = tid; idx < 256; idx += blockDim.x) {
+            const int ln = idx / 4, e = idx % 4;
             float g = 0.f, u = 0.f;
-            for (int w = 0; w < n_waves; ++w) {
-                g += red[(((w * MT + t) * RW + 0) * 64 + ln) * 4 + e];
-                u += red[(((w * MT + t) * RW + 1) * 64 + ln) * 4 + e];
+            for (int w = 0; w < k_waves; ++w) {
+                g += red[(w * 64 + ln) * 4 + e];
+                u += red[((k_waves + w) * 64 + ln) * 4 + e];
             }
-            const int m = t * 16 + ln % 16, col = blockIdx.x * 16 + 4 * (ln / 16) + e;
+            const int m = ln % 16, col = blockIdx.x * 16 + 4 * (ln / 16) + e;
             if (m < M && 2 * col < N) C[(size_t)m * (N / 2) + col] = from_float<TC>(u * (g / (1.0f + expf(-g))));
         }
         return;
@@ -366,15 +370,16 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
                                            int c_dtype, int n_waves, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23) || N % 32) return (int)hipErrorInvalidValue;
-    if (n_waves < 1 || n_waves > SK_MAX_WAVES) return (int)hipErrorInvalidValue;
-    const int k_per_wave = ((K + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
-    const int k_per_split = k_per_wave * n_waves;
+    if (n_waves < 2 || n_waves > SK_MAX_WAVES_SWIGLU || n_waves % 2) return (int)hipErrorInvalidValue;
+    const int k_waves = n_waves / 2;
+    const int k_per_wave = ((K + k_waves - 1) / k_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
+    const int k_per_split = k_per_wave * k_waves;
     if (c_dtype == 0)
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 2, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 1, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (float*)C, (float*)nullptr, M, N, K,
                            k_per_split, k_per_wave);
     else
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 2, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K,
                            k_per_split, k_per_wave);
     return soc_last_error();

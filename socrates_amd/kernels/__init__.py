@@ -91,7 +91,7 @@ class HipKernels:
         # torch.mm), as the reference's all do (nn.Linear); False keeps them on this
         # package's tiled MFMA kernel
         self.library_gemm = True
-        self._decode_blocks = None
+        self.swiglu_waves = 8           # waves of the fused gate+up product (measured: 4, 8, 16 within 5 %)
 
     # -- helpers -----------------------------------------------------------------------------
     def _stream(self):
@@ -189,8 +189,8 @@ class HipKernels:
             self._want(x, "x")
             self._want(w_gate_up, "weight", None, (N, K))
             out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
-            n_waves = 8
-            while n_waves > 1 and K // n_waves < 128:
+            n_waves = self.swiglu_waves          # half of them per tile (gate, up), splitting K
+            while n_waves > 2 and K // (n_waves // 2) < 128:
                 n_waves //= 2
             _check(self._gemm.soc_gemm_bf16_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(N),
                                                           c_int(K), c_int(self.code), c_int(n_waves),
@@ -343,17 +343,12 @@ class HipKernels:
 
     def _row_blocks(self, ctx, n_tokens, tokens_per_block):
         """int32 [blocks, 2] on the device: (first token, tokens) of each run of at most
-        ``tokens_per_block`` tokens of one sequence."""
+        ``tokens_per_block`` tokens of one sequence; None when every token is a run."""
         import numpy as np
         host = getattr(ctx, "host", None)
         if host is None or "seq_qstart" not in host or tokens_per_block == 1 or ctx.max_q_len == 1:
-            # every token alone (always right; what a decode step is anyway)
-            if self._decode_blocks is None:
-                # allocated once for the largest call: captured graphs keep its address
-                n = 65535
-                t = torch.stack([torch.arange(n, dtype=torch.int32), torch.ones(n, dtype=torch.int32)], 1)
-                self._decode_blocks = t.contiguous().to(self.device)
-            return self._decode_blocks[:n_tokens], n_tokens
+            # every token alone (always right; what a decode step is anyway): no list
+            return None, n_tokens
         cache = host.setdefault("row_blocks", {})
         if tokens_per_block not in cache:
             qstart = host["seq_qstart"].astype(np.int64)
