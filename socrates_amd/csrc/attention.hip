@@ -316,7 +316,9 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        float* __restrict__ part_ml, int Hq, int Hkv, int BS, float scale, int window,
                        int split_len, int n_splits, int group_pad_log2) {
     __shared__ __attribute__((aligned(16))) uint16_t v_lds[4][16 * V_STRIDE];
-    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    // the wave index is the same in all lanes: say so, and what depends on it (the task, its
+    // token, position and table row) is computed and loaded on the scalar side
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SOC_WAVE), lane = threadIdx.x % SOC_WAVE;
     const int G = Hq / Hkv;
     const int Gp = 1 << group_pad_log2;                 // rows per token in a row block
     const int chunks = (G + 15) / 16;                   // head chunks when G > 16
@@ -696,7 +698,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     static_assert(D <= 128, "one key pair per thread");
     __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][PF_K_ELEMS];
     __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][PF_V_ELEMS];
-    const int tid = threadIdx.x, wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int li = lane % 16, kb = lane / 16;
     const int G = Hq / Hkv, Gp = 1 << group_pad_log2;
     const int chunks = (G + 15) / 16;

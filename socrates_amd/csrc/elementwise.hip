@@ -332,12 +332,25 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                                     int rotary_dim, int BS, float eps, int heads_per_wave) {
     __shared__ float cos_t[SOC_MAX_HEAD / 2], sin_t[SOC_MAX_HEAD / 2];
     const int n = blockIdx.x;
-    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SOC_WAVE), lane = threadIdx.x % SOC_WAVE;
     const int heads = Hq + 2 * Hkv;
-    const int pos = positions ? positions[n] : 0;
     const int half = rotary_dim / 2;
     const int e0 = lane * VE;                          // this lane's elements e0 .. e0 + VE - 1
     const bool lane_on = e0 < D;                       // D is a multiple of VE
+    // A wave takes head after head (the same trip count for all waves); the next head's
+    // load is issued before the current one is worked on, and the first before anything
+    // that depends on the token's position.
+    auto load_head = [&](int it, float (&dst)[VE]) {
+        const int h = (blockIdx.y * heads_per_wave + it) * 4 + wave;
+        if (it < heads_per_wave && h < heads && lane_on) VecLoad<T, VE>::load(qkv + ((size_t)n * heads + h) * D + e0, dst);
+        else {
+#pragma unroll
+            for (int i = 0; i < VE; ++i) dst[i] = 0.f;
+        }
+    };
+    float v[VE], nxt[VE];
+    load_head(0, v);
+    const int pos = positions ? positions[n] : 0;
     if (inv_freq) {
         // the token's angles once per workgroup (float32, accurate range reduction:
         // positions reach thousands of radians)
@@ -349,55 +362,38 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
         const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
         page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;
     }
-    // Heads are taken HB at a time per wave (their loads are issued together). Measured on
-    // prompt portions of 2,048 tokens, one at a time is as fast as four.
-    constexpr int HB = 1;
-    for (int it0 = 0; it0 < heads_per_wave; it0 += HB) {          // the same trip count for all waves
-        float vv[HB][VE];
+    for (int it = 0; it < heads_per_wave; ++it) {
+        load_head(it + 1, nxt);
+        const int h = (blockIdx.y * heads_per_wave + it) * 4 + wave;
+        const bool active = h < heads;
+        const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
+        float ss = 0.f;
 #pragma unroll
-        for (int b = 0; b < HB; ++b) {
-            const int h = (blockIdx.y * heads_per_wave + it0 + b) * 4 + wave;
-            const bool on = it0 + b < heads_per_wave && h < heads && lane_on;
-            if (on) VecLoad<T, VE>::load(qkv + ((size_t)n * heads + h) * D + e0, vv[b]);
-            else {
+        for (int i = 0; i < VE; ++i) ss += v[i] * v[i];
+        const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
+        if (gain && active) {
+            ss = wave_sum(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
-                for (int i = 0; i < VE; ++i) vv[b][i] = 0.f;
-            }
+            for (int i = 0; i < VE; ++i) if (lane_on) v[i] = v[i] * inv * gain[e0 + i];
         }
+        if (inv_freq) {                                 // uniform over the wave
+            // the partner of element e is e +- half: the same slot of the lane half / VE away
+            // (half is a multiple of VE, checked by the launcher)
+            const int shift = half / VE;
+            const int src = e0 < half ? lane + shift : lane - shift;
 #pragma unroll
-        for (int b = 0; b < HB; ++b) {
-            if (it0 + b >= heads_per_wave) break;                   // uniform
-            const int h = (blockIdx.y * heads_per_wave + it0 + b) * 4 + wave;
-            const bool active = h < heads;
-            const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
-            float (&v)[VE] = vv[b];
-            float ss = 0.f;
-#pragma unroll
-            for (int i = 0; i < VE; ++i) ss += v[i] * v[i];
-            const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
-            if (gain && active) {
-                ss = wave_sum(ss);
-                const float inv = 1.0f / sqrtf(ss / (float)D + eps);
-#pragma unroll
-                for (int i = 0; i < VE; ++i) if (lane_on) v[i] = v[i] * inv * gain[e0 + i];
-            }
-            if (inv_freq) {                                 // uniform over the wave
-                // the partner of element e is e +- half: the same slot of the lane half / VE away
-                // (half is a multiple of VE, checked by the launcher)
-                const int shift = half / VE;
-                const int src = e0 < half ? lane + shift : lane - shift;
-#pragma unroll
-                for (int i = 0; i < VE; ++i) {
-                    const float partner = __shfl(v[i], src & (SOC_WAVE - 1), SOC_WAVE);
-                    const int e = e0 + i;
-                    if (active && (is_q || is_k) && lane_on && e < rotary_dim) {
-                        const int j = e < half ? e : e - half;
-                        const float sn = sin_t[j], cs = cos_t[j];
-                        v[i] = e < half ? v[i] * cs - partner * sn : v[i] * cs + partner * sn;
-                    }
+            for (int i = 0; i < VE; ++i) {
+                const float partner = __shfl(v[i], src & (SOC_WAVE - 1), SOC_WAVE);
+                const int e = e0 + i;
+                if (active && (is_q || is_k) && lane_on && e < rotary_dim) {
+                    const int j = e < half ? e : e - half;
+                    const float sn = sin_t[j], cs = cos_t[j];
+                    v[i] = e < half ? v[i] * cs - partner * sn : v[i] * cs + partner * sn;
                 }
             }
-            if (!active || !lane_on) continue;
+        }
+        if (active && lane_on) {
             T* dst;
             if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
             else {
@@ -410,8 +406,7 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
             } else if constexpr (sizeof(T) == 2) {
                 uint32_t pk[VE / 2];
 #pragma unroll
-                for (int i = 0; i < VE / 2; ++i)
-                    pk[i] = (uint32_t)f32_to_bf16_bits(v[2 * i]) | ((uint32_t)f32_to_bf16_bits(v[2 * i + 1]) << 16);
+                for (int i = 0; i < VE / 2; ++i) pk[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
                 if constexpr (VE == 2) *reinterpret_cast<uint32_t*>(dst + e0) = pk[0];
                 else *reinterpret_cast<uint2*>(dst + e0) = make_uint2(pk[0], pk[1]);
             } else {
@@ -419,6 +414,8 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
                 for (int i = 0; i < VE; ++i) dst[e0 + i] = from_float<T>(v[i]);
             }
         }
+#pragma unroll
+        for (int i = 0; i < VE; ++i) v[i] = nxt[i];
     }
 }
 
