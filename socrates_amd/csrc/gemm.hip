@@ -390,12 +390,13 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
 // [M <= 64] x [N, K] product.
 SOC_EXPORT void soc_gemm_skinny_plan(int M, int N, int K, int allow_split, int* row_tiles, int* n_waves,
                                      int* k_splits) {
-    // From measurements at K = 2560..9728 on an MI355X: wide outputs have enough row tiles
-    // to fill the GPU with one tile per workgroup; narrow ones need two workgroups per K.
+    // From measurements on an MI355X at the products of 4B-, 8B- and 32B-sized layers
+    // (N 2560..51200, K 2560..25600): one tile per workgroup and eight waves over K is within
+    // a few per cent of the best everywhere from N = 4096 on; a long K over a middling N gains
+    // from two workgroups per tile; narrow outputs need that to fill the GPU.
     int rw, nw, ks = 1;
     if (M > 16) { rw = 2; nw = N >= 16384 ? 4 : 8; }
-    else if (N >= 16384) { rw = 1; nw = 8; }
-    else if (N >= 4096) { rw = 2; nw = 4; }
+    else if (N >= 4096) { rw = 1; nw = 8; if (allow_split && K >= 8192 && N < 16384) ks = 2; }
     else if (allow_split && K >= 2048) { rw = 2; nw = 8; ks = 2; }
     else { rw = 1; nw = 8; }
     while (nw > 1 && K / (nw * ks) < 128) nw /= 2;
