@@ -533,7 +533,7 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
     __shared__ __attribute__((aligned(16))) float4 red[SOC_WAVE];
     const int h = blockIdx.x, n = blockIdx.y, lane = threadIdx.x;
     const size_t base = ((size_t)n * Hq + h) * n_splits;
-    constexpr int FAST = 16;                                // partials a lane holds on the short path
+    constexpr int FAST = 32;                                // partials a lane holds on the short path
     if (n_splits <= SOC_WAVE && n_splits <= FAST * NG) {
         // Few splits: every load is issued before any is needed (one trip to memory instead
         // of two). An empty split's partial was never written: it is loaded, but not used.
