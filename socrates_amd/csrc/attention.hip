@@ -306,15 +306,16 @@ __device__ __forceinline__ uint4 load_qk_slice(const bf16* row, int kk, int kb) 
     }
 }
 
-template <int RT>
+// TP: pages hold a multiple of 16 keys (and a power of two of them), so a tile lies in one page.
+template <int RT, bool TP>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                        const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
                        int table_width, const int* __restrict__ token_rows,
                        const int* __restrict__ positions, const int* __restrict__ row_blocks,
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
-                       float* __restrict__ part_ml, int Hq, int Hkv, int BS, float scale, int window,
-                       int split_len, int n_splits, int group_pad_log2) {
+                       float* __restrict__ part_ml, int Hq, int Hkv, int BS, int bs_shift, float scale,
+                       int window, int split_len, int n_splits, int group_pad_log2) {
     __shared__ __attribute__((aligned(16))) uint16_t v_lds[4][16 * V_STRIDE];
     // the wave index is the same in all lanes: say so, and what depends on it (the task, its
     // token, position and table row) is computed and loaded on the scalar side
@@ -366,19 +367,64 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     }
 
+    const float c2 = scale * 1.44269504088896340736f;   // scores to base 2
+    const size_t page_stride = (size_t)Hkv * BS * D;
+    const bf16* k_base = k_pool + (size_t)kvh * BS * D;
+    const bf16* v_base = v_pool + (size_t)kvh * BS * D;
+    // Pages of a multiple of 16 keys: a tile lies in one page, so its page is one value for
+    // the whole wave, read on the scalar side, and no lane needs another's.
+    constexpr bool tile_in_page = TP;
     // Page of this lane's key of a tile (lanes 0..15 of every lane group hold keys 0..15).
     // Keys that no row of the block can see get page -1 and are never read.
     auto lookup = [&](int key0) -> int {
-        const int key = key0 + li;
-        return (key >= kmin && key < khi) ? table[key / BS] : -1;
+        if constexpr (tile_in_page) {
+            // the tile's page, if any of its keys is read (the same in all lanes)
+            const bool any = key0 < khi && key0 + 16 > kmin;
+            return any ? table[__builtin_amdgcn_readfirstlane(key0 >> bs_shift)] : -1;
+        } else {
+            const int key = key0 + li;
+            return (key >= kmin && key < khi) ? table[key / BS] : -1;
+        }
     };
     // Global loads of one tile: this lane's K slices and its share of the V tile. Zeros
     // stand in for keys that are not read, so that whatever lies in stale slots or in the
     // null page (inf, NaN) never meets a product.
     auto fetch = [&](int key0, int page, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
         const int key = key0 + li;
+        if constexpr (tile_in_page) {
+            if (page < 0) {                                  // uniform: nothing of the tile is read
+#pragma unroll
+                for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+                for (int j = 0; j < V_PER_LANE; ++j) vr[j] = make_uint4(0u, 0u, 0u, 0u);
+                return;
+            }
+            const size_t tile_off = (size_t)page * page_stride + (size_t)((key0 & (BS - 1)) * D);
+            const bf16* krow = k_base + tile_off + li * D;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int c = lane + 64 * j;
+                const int vk = (c / (D / 8)) & 15, part = c % (D / 8);
+                vr[j] = (V_CHUNKS % 64 == 0 || c < V_CHUNKS)
+                            ? *reinterpret_cast<const uint4*>(v_base + tile_off + vk * D + part * 8)
+                            : make_uint4(0u, 0u, 0u, 0u);
+            }
+            if (key0 < kmin || key0 + 16 > khi) {            // uniform: a tile at an edge of the range
+                const bool ok = key >= kmin && key < khi;
+#pragma unroll
+                for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+                for (int j = 0; j < V_PER_LANE; ++j) {
+                    const int vkey = key0 + (((lane + 64 * j) / (D / 8)) & 15);
+                    vr[j] = (vkey >= kmin && vkey < khi) ? vr[j] : make_uint4(0u, 0u, 0u, 0u);
+                }
+            }
+            return;
+        } else {
         if (page >= 0) {
-            const bf16* krow = k_pool + ((size_t)page * Hkv * BS + (size_t)kvh * BS + key % BS) * D;
+            const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key % BS) * D;
 #pragma unroll
             for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
         } else {
@@ -392,14 +438,17 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
             if ((V_CHUNKS % 64 == 0 || c < V_CHUNKS) && vpage >= 0)
                 vr[j] = *reinterpret_cast<const uint4*>(
-                    v_pool + ((size_t)vpage * Hkv * BS + (size_t)kvh * BS + (key0 + vk) % BS) * D + part * 8);
+                    v_base + (size_t)vpage * page_stride + (size_t)((key0 + vk) % BS) * D + part * 8);
             else
                 vr[j] = make_uint4(0u, 0u, 0u, 0u);
         }
+        }
     };
 
-    // One tile: V to LDS, scores, online softmax, weighted values.
-    auto compute = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE]) {
+    // One tile: V to LDS, scores, online softmax, weighted values. MASKED: some key of the
+    // tile is hidden from some row of the block (or lies outside the split).
+    auto compute = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE], auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
         // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk)
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
@@ -424,29 +473,31 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             float mx = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key = key0 + 4 * kb + r;
-                bool seen = key <= row_pos[rt] && key < khi && key >= split * split_len;
-                if (window > 0) seen = seen && key > row_pos[rt] - window;
-                sv[r] = seen ? s[r] * scale : -INFINITY;
+                sv[r] = s[r] * c2;
+                if constexpr (MASKED) {
+                    const int key = key0 + 4 * kb + r;
+                    bool seen = key <= row_pos[rt] && key < khi && key >= split * split_len;
+                    if (window > 0) seen = seen && key > row_pos[rt] - window;
+                    sv[r] = seen ? sv[r] : -INFINITY;
+                }
                 mx = fmaxf(mx, sv[r]);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
+            mx = max_xor32(max_xor16(mx));
             const float mn = fmaxf(m[rt], mx);
-            const float ms = mn == -INFINITY ? 0.f : mn;
-            alpha[rt] = __expf(m[rt] - ms);
+            const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
+            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - ms);
+            float p[4];
             float psum = 0.f;
-            uint16_t pb[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float p = __expf(sv[r] - ms);
-                psum += p;
-                pb[r] = f32_to_bf16_bits(p);
+                p[r] = __builtin_amdgcn_exp2f(sv[r] - ms);
+                psum += p[r];
             }
             l[rt] = l[rt] * alpha[rt] + psum;
             any_rescale = any_rescale || (m[rt] != mn);
             m[rt] = mn;
-            pf[rt] = (s16x4_t){(short)pb[0], (short)pb[1], (short)pb[2], (short)pb[3]};
+            const uint32_t p01 = pack_bf16x2(p[0], p[1]), p23 = pack_bf16x2(p[2], p[3]);
+            pf[rt] = (s16x4_t){(short)(p01 & 0xffffu), (short)(p01 >> 16), (short)(p23 & 0xffffu), (short)(p23 >> 16)};
         }
         if (__any(any_rescale)) {
 #pragma unroll
@@ -466,6 +517,19 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         }
         __builtin_amdgcn_wave_barrier();
     };
+    // whole: every key of the tile lies in the split, at or before the block's first position
+    // and inside the window of its last one, so no score needs a mask
+    const int last_pos = pos0 + ntok - 1;
+    auto tile = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE]) {
+        const bool whole = key0 >= split * split_len && key0 + 15 < khi && key0 + 15 <= pos0 &&
+                           (window <= 0 || key0 > last_pos - window);
+        if constexpr (D > 128) {
+            compute(key0, kf, vr, std::true_type{});         // one variant: registers are short at these sizes
+        } else {
+            if (whole) compute(key0, kf, vr, std::false_type{});
+            else compute(key0, kf, vr, std::true_type{});
+        }
+    };
 
     // Three tiles are in flight per wave (48 keys): HBM latency is several times the time one
     // tile takes to compute. Buffer b holds tiles b, b + 3, b + 6, ... of the wave's range;
@@ -480,13 +544,13 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     if (klo + 64 < khi) pg1 = lookup(klo + 64);
     if (klo + 80 < khi) pg2 = lookup(klo + 80);
     for (int key0 = klo; key0 < khi; key0 += 48) {
-        compute(key0, kf0, vr0);
+        tile(key0, kf0, vr0);
         if (key0 + 48 < khi) { fetch(key0 + 48, pg0, kf0, vr0); pg0 = lookup(key0 + 96); }
         if (key0 + 16 >= khi) break;
-        compute(key0 + 16, kf1, vr1);
+        tile(key0 + 16, kf1, vr1);
         if (key0 + 64 < khi) { fetch(key0 + 64, pg1, kf1, vr1); pg1 = lookup(key0 + 112); }
         if (key0 + 32 >= khi) break;
-        compute(key0 + 32, kf2, vr2);
+        tile(key0 + 32, kf2, vr2);
         if (key0 + 80 < khi) { fetch(key0 + 80, pg2, kf2, vr2); pg2 = lookup(key0 + 128); }
     }
 
@@ -494,8 +558,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         float L = l[rt];
-        L += __shfl_xor(L, 16, SOC_WAVE);
-        L += __shfl_xor(L, 32, SOC_WAVE);
+        L = sum_xor32(sum_xor16(L));
         if (row_pos[rt] < 0) continue;
         const size_t base = row_q[rt];                                   // (token * Hq + head) * D
         if (n_splits == 1) {
@@ -549,7 +612,7 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
                        : make_float4(0.f, 0.f, 0.f, 0.f);
         }
         const float M = wave_max(ms);
-        const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+        const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);   // the maxima are in base 2
         const float L = wave_sum(w * ls);
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -585,7 +648,7 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
     float lsum = 0.f;                                       // the launcher allows at most 256 splits
     for (int s = lane; s < n_splits; s += SOC_WAVE) {
         const float ms = part_ml[(base + s) * 2];
-        const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+        const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
         weight[s] = w;
         lsum += w * part_ml[(base + s) * 2 + 1];
     }
@@ -642,17 +705,32 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     if (n_splits > 256) return (int)hipErrorInvalidValue;        // the merge holds 256 weights
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     const dim3 grid((unsigned)((tasks + 3) / 4), n_splits);
+    int bs_shift = -1;                                           // log2 of the page size if it is a power of two
+    if ((BS & (BS - 1)) == 0)
+        for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
-        token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, Hq, Hkv, BS, scale, \
-        window, split_len, n_splits, group_pad_log2
-    if (row_tiles == 1)
-        hipLaunchKernelGGL(paged_attn_mfma_kernel<1>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
-    else if (row_tiles == 2)
-        hipLaunchKernelGGL(paged_attn_mfma_kernel<2>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
-    else if (row_tiles == 4)
-        hipLaunchKernelGGL(paged_attn_mfma_kernel<4>, grid, dim3(256), 0, stream, SOC_MFMA_ARGS);
-    else
+        token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, Hq, Hkv, BS, bs_shift, \
+        scale, window, split_len, n_splits, group_pad_log2
+    // Row tiles beyond what the registers hold at this head size are refused: two up to head
+    // size 128, four up to 64.
+    const bool tp = bs_shift >= 4;
+#define SOC_MFMA_LAUNCH(RT_)                                                                          \
+    do {                                                                                              \
+        if (tp) hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, true>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS); \
+        else hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, false>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS);   \
+    } while (0)
+    if (row_tiles == 1) {
+        SOC_MFMA_LAUNCH(1);
+    } else if (row_tiles == 2) {
+        if constexpr (D <= 128) SOC_MFMA_LAUNCH(2);
+        else return (int)hipErrorInvalidValue;
+    } else if (row_tiles == 4) {
+        if constexpr (D <= 64) SOC_MFMA_LAUNCH(4);
+        else return (int)hipErrorInvalidValue;
+    } else {
         return (int)hipErrorInvalidValue;
+    }
+#undef SOC_MFMA_LAUNCH
 #undef SOC_MFMA_ARGS
     int err = soc_last_error();
     if (err || n_splits == 1) return err;
@@ -839,8 +917,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                 }
                 mx = fmaxf(mx, t[r]);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16, SOC_WAVE));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, SOC_WAVE));
+            mx = max_xor32(max_xor16(mx));
             const float mn = fmaxf(m[rt], mx);
             const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
             alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - ms);
@@ -924,8 +1001,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         float L = l[rt];
-        L += __shfl_xor(L, 16, SOC_WAVE);
-        L += __shfl_xor(L, 32, SOC_WAVE);
+        L = sum_xor32(sum_xor16(L));
         if (row_pos[rt] < 0) continue;
         const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll

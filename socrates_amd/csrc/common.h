@@ -90,16 +90,42 @@ template <int N> struct VecLoad<bf16, N> {
     }
 };
 
+// Cross-lane steps of a wave reduction without a trip through LDS: within a row of 16
+// lanes DPP operands (lane ^ 1, lane ^ 2, then the mirror images of a half row and of a
+// row, which pair groups whose lanes already agree), across rows the gfx950 lane-swap
+// instructions. Every step combines a pair symmetrically, so all lanes end with the same bits.
+template <int CTRL> __device__ __forceinline__ float soc_dpp(float v) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int SOC_DPP_XOR1 = 0xB1, SOC_DPP_XOR2 = 0x4E, SOC_DPP_HALF_MIRROR = 0x141, SOC_DPP_ROW_MIRROR = 0x140;
+
+typedef uint32_t soc_u32x2 __attribute__((ext_vector_type(2)));
+// this lane's value and that of lane ^ 16 (in some order)
+__device__ __forceinline__ soc_u32x2 soc_pair_xor16(float v) {
+    return __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+}
+__device__ __forceinline__ soc_u32x2 soc_pair_xor32(float v) {
+    return __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+}
+__device__ __forceinline__ float sum_xor16(float v) { const soc_u32x2 p = soc_pair_xor16(v); return __uint_as_float(p.x) + __uint_as_float(p.y); }
+__device__ __forceinline__ float sum_xor32(float v) { const soc_u32x2 p = soc_pair_xor32(v); return __uint_as_float(p.x) + __uint_as_float(p.y); }
+__device__ __forceinline__ float max_xor16(float v) { const soc_u32x2 p = soc_pair_xor16(v); return fmaxf(__uint_as_float(p.x), __uint_as_float(p.y)); }
+__device__ __forceinline__ float max_xor32(float v) { const soc_u32x2 p = soc_pair_xor32(v); return fmaxf(__uint_as_float(p.x), __uint_as_float(p.y)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = SOC_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, SOC_WAVE);
-    return v;
+    v += soc_dpp<SOC_DPP_XOR1>(v);
+    v += soc_dpp<SOC_DPP_XOR2>(v);
+    v += soc_dpp<SOC_DPP_HALF_MIRROR>(v);
+    v += soc_dpp<SOC_DPP_ROW_MIRROR>(v);
+    return sum_xor32(sum_xor16(v));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int m = SOC_WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, SOC_WAVE));
-    return v;
+    v = fmaxf(v, soc_dpp<SOC_DPP_XOR1>(v));
+    v = fmaxf(v, soc_dpp<SOC_DPP_XOR2>(v));
+    v = fmaxf(v, soc_dpp<SOC_DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, soc_dpp<SOC_DPP_ROW_MIRROR>(v));
+    return max_xor32(max_xor16(v));
 }
 
 // Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024); every

@@ -412,6 +412,7 @@ class HipKernels:
                     "paged_attention (prefill)")
                 return out
             rt = self.attention_row_tiles or 1
+            rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
             tokens_per_block = max(1, (16 * rt) >> gpl)
             blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
             split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
