@@ -374,74 +374,50 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     // Pages of a multiple of 16 keys: a tile lies in one page, so its page is one value for
     // the whole wave, read on the scalar side, and no lane needs another's.
     constexpr bool tile_in_page = TP;
-    // Page of this lane's key of a tile (lanes 0..15 of every lane group hold keys 0..15).
-    // Keys that no row of the block can see get page -1 and are never read.
+    // Loads must stay in flight until their tile is computed, so nothing touches what they
+    // bring before that: no branch around a load (the two sides would have to be reconciled
+    // in registers behind it), no select on its result. A key that must not be read (outside
+    // what the block's rows can see) is redirected to the first entry of the row's table (a
+    // page of the pool whatever it holds), and its data are replaced by zeros when the tile
+    // is computed, so that what lies in stale slots (inf, NaN) never meets a product.
+    // lookup: the page of the tile (TP: one value for the wave) or of this lane's key (lanes
+    // 0..15 of every lane group hold keys 0..15).
     auto lookup = [&](int key0) -> int {
         if constexpr (tile_in_page) {
-            // the tile's page, if any of its keys is read (the same in all lanes)
             const bool any = key0 < khi && key0 + 16 > kmin;
-            return any ? table[__builtin_amdgcn_readfirstlane(key0 >> bs_shift)] : -1;
+            return table[__builtin_amdgcn_readfirstlane(any ? key0 >> bs_shift : 0)];
         } else {
             const int key = key0 + li;
-            return (key >= kmin && key < khi) ? table[key / BS] : -1;
+            const bool ok = key >= kmin && key < khi;
+            return table[ok ? key / BS : 0];
         }
     };
-    // Global loads of one tile: this lane's K slices and its share of the V tile. Zeros
-    // stand in for keys that are not read, so that whatever lies in stale slots or in the
-    // null page (inf, NaN) never meets a product.
+    // Global loads of one tile: this lane's K slices and its share of the V tile.
     auto fetch = [&](int key0, int page, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
-        const int key = key0 + li;
         if constexpr (tile_in_page) {
-            if (page < 0) {                                  // uniform: nothing of the tile is read
-#pragma unroll
-                for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-                for (int j = 0; j < V_PER_LANE; ++j) vr[j] = make_uint4(0u, 0u, 0u, 0u);
-                return;
-            }
             const size_t tile_off = (size_t)page * page_stride + (size_t)((key0 & (BS - 1)) * D);
             const bf16* krow = k_base + tile_off + li * D;
 #pragma unroll
             for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
 #pragma unroll
             for (int j = 0; j < V_PER_LANE; ++j) {
-                const int c = lane + 64 * j;
-                const int vk = (c / (D / 8)) & 15, part = c % (D / 8);
-                vr[j] = (V_CHUNKS % 64 == 0 || c < V_CHUNKS)
-                            ? *reinterpret_cast<const uint4*>(v_base + tile_off + vk * D + part * 8)
-                            : make_uint4(0u, 0u, 0u, 0u);
+                const int c = (lane + 64 * j) % V_CHUNKS;        // lanes past the tile's chunks reload one of them
+                const int vk = c / (D / 8), part = c % (D / 8);
+                vr[j] = *reinterpret_cast<const uint4*>(v_base + tile_off + vk * D + part * 8);
             }
-            if (key0 < kmin || key0 + 16 > khi) {            // uniform: a tile at an edge of the range
-                const bool ok = key >= kmin && key < khi;
-#pragma unroll
-                for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-                for (int j = 0; j < V_PER_LANE; ++j) {
-                    const int vkey = key0 + (((lane + 64 * j) / (D / 8)) & 15);
-                    vr[j] = (vkey >= kmin && vkey < khi) ? vr[j] : make_uint4(0u, 0u, 0u, 0u);
-                }
-            }
-            return;
         } else {
-        if (page >= 0) {
+            const int key = key0 + li;
             const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key % BS) * D;
 #pragma unroll
             for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
-        } else {
 #pragma unroll
-            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = make_uint4(0u, 0u, 0u, 0u);
-        }
-#pragma unroll
-        for (int j = 0; j < V_PER_LANE; ++j) {
-            const int c = lane + 64 * j;
-            const int vk = (c / (D / 8)) & 15, part = c % (D / 8);
-            const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
-            if ((V_CHUNKS % 64 == 0 || c < V_CHUNKS) && vpage >= 0)
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int c = (lane + 64 * j) % V_CHUNKS;
+                const int vk = c / (D / 8), part = c % (D / 8);
+                const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
                 vr[j] = *reinterpret_cast<const uint4*>(
                     v_base + (size_t)vpage * page_stride + (size_t)((key0 + vk) % BS) * D + part * 8);
-            else
-                vr[j] = make_uint4(0u, 0u, 0u, 0u);
-        }
+            }
         }
     };
 
@@ -449,18 +425,25 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     // tile is hidden from some row of the block (or lies outside the split).
     auto compute = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk)
+        // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk); keys
+        // that were not to be read become zeros here, now that their loads have landed
 #pragma unroll
         for (int j = 0; j < V_PER_LANE; ++j) {
             const int c = lane + 64 * j;
             if (V_CHUNKS % 64 == 0 || c < V_CHUNKS) {
                 const int vk = c / (D / 8), part = c % (D / 8);
+                uint4 t = vr[j];
+                if constexpr (MASKED) {
+                    const int vkey = key0 + vk;
+                    if (vkey < kmin || vkey >= khi) t = make_uint4(0u, 0u, 0u, 0u);
+                }
                 uint2* dst = reinterpret_cast<uint2*>(&vl[vk * V_STRIDE + part * 8]);
-                dst[0] = make_uint2(vr[j].x, vr[j].y);
-                dst[1] = make_uint2(vr[j].z, vr[j].w);
+                dst[0] = make_uint2(t.x, t.y);
+                dst[1] = make_uint2(t.z, t.w);
             }
         }
         __builtin_amdgcn_wave_barrier();
+        const bool k_ok = !MASKED || (key0 + li >= kmin && key0 + li < khi);
         s16x4_t pf[RT];
         bool any_rescale = false;
         float alpha[RT];
@@ -468,7 +451,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         for (int rt = 0; rt < RT; ++rt) {
             f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < QK_STEPS; ++kk) s = qk_mfma(kf.v[kk], qf[rt][kk], s);
+            for (int kk = 0; kk < QK_STEPS; ++kk)
+                s = qk_mfma(k_ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u), qf[rt][kk], s);
             float sv[4];
             float mx = -INFINITY;
 #pragma unroll
@@ -531,28 +515,41 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         }
     };
 
-    // Three tiles are in flight per wave (48 keys): HBM latency is several times the time one
-    // tile takes to compute. Buffer b holds tiles b, b + 3, b + 6, ... of the wave's range;
-    // the page of a tile is looked up three steps before its loads are issued.
+    // Three tiles are in flight per wave (48 keys). Buffer b holds tiles b, b + 3, b + 6, ...
+    // of the wave's range; the page of a tile is looked up three tiles before its loads are
+    // issued.
     KFrag kf0, kf1, kf2;
     uint4 vr0[V_PER_LANE], vr1[V_PER_LANE], vr2[V_PER_LANE];
-    int pg0 = -1, pg1 = -1, pg2 = -1;
-    if (klo < khi) fetch(klo, lookup(klo), kf0, vr0);
-    if (klo + 16 < khi) fetch(klo + 16, lookup(klo + 16), kf1, vr1);
-    if (klo + 32 < khi) fetch(klo + 32, lookup(klo + 32), kf2, vr2);
-    if (klo + 48 < khi) pg0 = lookup(klo + 48);
-    if (klo + 64 < khi) pg1 = lookup(klo + 64);
-    if (klo + 80 < khi) pg2 = lookup(klo + 80);
-    for (int key0 = klo; key0 < khi; key0 += 48) {
+    // Lookups first, then the tile loads: a wait for a lookup then leaves the loads in flight.
+    // Lookups may run past the end of the range (redirected); tile loads do not: the rounds
+    // of the main loop are those in which all three buffers have a tile to load, and what
+    // remains (at most five tiles, two of them still to load) follows without a loop.
+    int pa = lookup(klo), pb = lookup(klo + 16), pc = lookup(klo + 32);
+    int pg0 = lookup(klo + 48), pg1 = lookup(klo + 64), pg2 = lookup(klo + 80);
+    fetch(klo, pa, kf0, vr0);
+    if (klo + 16 < khi) fetch(klo + 16, pb, kf1, vr1);
+    if (klo + 32 < khi) fetch(klo + 32, pc, kf2, vr2);
+    int key0 = klo;
+    for (; key0 + 80 < khi; key0 += 48) {
         tile(key0, kf0, vr0);
-        if (key0 + 48 < khi) { fetch(key0 + 48, pg0, kf0, vr0); pg0 = lookup(key0 + 96); }
-        if (key0 + 16 >= khi) break;
+        fetch(key0 + 48, pg0, kf0, vr0);
+        pg0 = lookup(key0 + 96);
         tile(key0 + 16, kf1, vr1);
-        if (key0 + 64 < khi) { fetch(key0 + 64, pg1, kf1, vr1); pg1 = lookup(key0 + 112); }
-        if (key0 + 32 >= khi) break;
+        fetch(key0 + 64, pg1, kf1, vr1);
+        pg1 = lookup(key0 + 112);
         tile(key0 + 32, kf2, vr2);
-        if (key0 + 80 < khi) { fetch(key0 + 80, pg2, kf2, vr2); pg2 = lookup(key0 + 128); }
+        fetch(key0 + 80, pg2, kf2, vr2);
+        pg2 = lookup(key0 + 128);
     }
+    tile(key0, kf0, vr0);
+    if (key0 + 48 < khi) fetch(key0 + 48, pg0, kf0, vr0);
+    if (key0 + 16 < khi) {
+        tile(key0 + 16, kf1, vr1);
+        if (key0 + 64 < khi) fetch(key0 + 64, pg1, kf1, vr1);
+    }
+    if (key0 + 32 < khi) tile(key0 + 32, kf2, vr2);
+    if (key0 + 48 < khi) tile(key0 + 48, kf0, vr0);
+    if (key0 + 64 < khi) tile(key0 + 64, kf1, vr1);
 
     // finish: the row sum is spread over the four lanes of the row's column
 #pragma unroll
