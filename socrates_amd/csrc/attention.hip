@@ -821,55 +821,47 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // Cooperative tile loads: a thread owns two neighbouring keys (2 kp, 2 kp + 1) and one
     // 16-byte part of them, of K and of V. Keys that no row of the block sees are never read;
     // zeros stand in for them.
+    // Loads must stay in flight until their tile is moved to LDS, so nothing touches what
+    // they bring before that: no branch around a load, no select on its result. A key that
+    // must not be read is redirected to the first entry of the row's table (a page of the
+    // pool whatever it holds) and becomes zeros when the tile is stored to LDS. Threads past
+    // the parts of a key (head sizes under 128) load a part again and store nothing.
     const int kp = tid % 16, part = tid / 16;
     const bool loader = part < PF_PARTS;
+    const int part_ld = PF_PARTS == 16 ? part : part % PF_PARTS;
     const size_t page_stride = (size_t)Hkv * BS * D;
-    const bf16* k_base = k_pool + (size_t)kvh * BS * D + part * 8;
-    const bf16* v_base = v_pool + (size_t)kvh * BS * D + part * 8;
-    const bool pair_in_page = bs_shift >= 1;           // keys 2 kp and 2 kp + 1 share a page
-    // a tile inside [kmin, khi) needs no predicate
+    const bf16* k_base = k_pool + (size_t)kvh * BS * D + part_ld * 8;
+    const bf16* v_base = v_pool + (size_t)kvh * BS * D + part_ld * 8;
     auto lookup = [&](int key0, int (&pg)[2]) {
-        if (!loader) { pg[0] = pg[1] = -1; return; }
-        if (pair_in_page && key0 >= kmin && key0 + PF_KEYS <= khi) {
-            pg[0] = pg[1] = table[(key0 + 2 * kp) >> bs_shift];
-            return;
-        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int key = key0 + 2 * kp + h;
-            pg[h] = (key >= kmin && key < khi) ? table[bs_shift >= 0 ? key >> bs_shift : key / BS] : -1;
+            const bool ok = key >= kmin && key < khi;
+            pg[h] = table[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
         }
     };
     auto fetch = [&](int key0, const int (&pg)[2], uint4 (&kr)[2], uint4 (&vr)[2]) {
-        if (!loader) return;
-        if (pair_in_page && key0 >= kmin && key0 + PF_KEYS <= khi) {
-            const size_t off = (size_t)pg[0] * page_stride + (size_t)(((key0 + 2 * kp) & (BS - 1)) * D);
-            kr[0] = *reinterpret_cast<const uint4*>(k_base + off);
-            kr[1] = *reinterpret_cast<const uint4*>(k_base + off + D);
-            vr[0] = *reinterpret_cast<const uint4*>(v_base + off);
-            vr[1] = *reinterpret_cast<const uint4*>(v_base + off + D);
-            return;
-        }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int key = key0 + 2 * kp + h;
-            if (pg[h] >= 0) {
-                const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
-                const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
-                kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
-                vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
-            } else {
-                kr[h] = make_uint4(0u, 0u, 0u, 0u);
-                vr[h] = make_uint4(0u, 0u, 0u, 0u);
-            }
+            const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
+            const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
+            kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
+            vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
         }
     };
-    auto stash = [&](int buf, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
+    auto stash = [&](int buf, int key0, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
         if (!loader) return;
-        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp) * PF_K_STRIDE + part * 8]) = kr[0];
-        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp + 1) * PF_K_STRIDE + part * 8]) = kr[1];
-        const uint32_t a[4] = {vr[0].x, vr[0].y, vr[0].z, vr[0].w};
-        const uint32_t b[4] = {vr[1].x, vr[1].y, vr[1].z, vr[1].w};
+        uint4 k0 = kr[0], k1 = kr[1], v0 = vr[0], v1 = vr[1];
+        if (key0 < kmin || key0 + PF_KEYS > khi) {           // uniform: a tile at an edge of the range
+            const int key = key0 + 2 * kp;
+            if (key < kmin || key >= khi) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
+            if (key + 1 < kmin || key + 1 >= khi) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
+        }
+        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp) * PF_K_STRIDE + part * 8]) = k0;
+        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp + 1) * PF_K_STRIDE + part * 8]) = k1;
+        const uint32_t a[4] = {v0.x, v0.y, v0.z, v0.w};
+        const uint32_t b[4] = {v1.x, v1.y, v1.z, v1.w};
         uint32_t* vt = reinterpret_cast<uint32_t*>(&v_lds[buf][(part * 8) * PF_V_STRIDE + 2 * kp]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -959,7 +951,11 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // their way into one pair of staging registers, and the pages of tile t + 2 were asked
     // for. The iteration issues the lookup of tile t + 3 and the loads of tile t + 2, computes,
     // and then moves tile t + 1 from its registers to the other LDS buffer, which nobody has
-    // read since the barrier that ended the previous iteration.
+    // read since the barrier that ended the previous iteration. Loads return in order, so a
+    // lookup is issued before the tile loads of its iteration: waiting for it then leaves
+    // those in flight. Lookups may run past the end of the range (redirected); tile loads do
+    // not: the main loop takes the rounds in which both buffers have a tile to load, and
+    // the last tiles (at most three) follow without a loop.
     auto tile = [&](int key0, int buf) {
         if (wave_has_rows && key0 <= wave_hi_pos) {
             // whole: every key of the tile is at or before the wave's first position and inside
@@ -970,29 +966,40 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             else compute(key0, buf, std::true_type{});
         }
     };
-    // Loads return in order, so a lookup is issued before the tile loads of its iteration:
-    // waiting for it then leaves those tile loads in flight.
     int pg0[2], pg1[2];
     uint4 kr0[2], vr0[2], kr1[2], vr1[2];
     lookup(klo, pg0);
     lookup(klo + PF_KEYS, pg1);
     fetch(klo, pg0, kr0, vr0);
     lookup(klo + 2 * PF_KEYS, pg0);
-    fetch(klo + PF_KEYS, pg1, kr1, vr1);
-    stash(0, kr0, vr0);
+    if (klo + PF_KEYS < khi) fetch(klo + PF_KEYS, pg1, kr1, vr1);
+    stash(0, klo, kr0, vr0);
     __syncthreads();
-    for (int key0 = klo; key0 < khi; key0 += 2 * PF_KEYS) {
+    int key0 = klo;
+    for (; key0 + 3 * PF_KEYS < khi; key0 += 2 * PF_KEYS) {
         lookup(key0 + 3 * PF_KEYS, pg1);
         fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
         tile(key0, 0);
-        stash(1, kr1, vr1);
+        stash(1, key0 + PF_KEYS, kr1, vr1);
         __syncthreads();
-        if (key0 + PF_KEYS >= khi) break;
         lookup(key0 + 4 * PF_KEYS, pg0);
         fetch(key0 + 3 * PF_KEYS, pg1, kr1, vr1);
         tile(key0 + PF_KEYS, 1);
-        stash(0, kr0, vr0);
+        stash(0, key0 + 2 * PF_KEYS, kr0, vr0);
         __syncthreads();
+    }
+    const bool has1 = key0 + PF_KEYS < khi, has2 = key0 + 2 * PF_KEYS < khi;      // the same in all threads
+    if (has2) fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
+    tile(key0, 0);
+    if (has1) {
+        stash(1, key0 + PF_KEYS, kr1, vr1);
+        __syncthreads();
+        tile(key0 + PF_KEYS, 1);
+        if (has2) {
+            stash(0, key0 + 2 * PF_KEYS, kr0, vr0);
+            __syncthreads();
+            tile(key0 + 2 * PF_KEYS, 0);
+        }
     }
 
 #pragma unroll
