@@ -340,13 +340,11 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
     // A wave takes head after head (the same trip count for all waves); the next head's
     // load is issued before the current one is worked on, and the first before anything
     // that depends on the token's position.
+    // (No branch around the load and nothing done to its result here, or the wave would wait
+    // for it on the spot: a head or a lane outside reads a valid address and is dropped later.)
     auto load_head = [&](int it, float (&dst)[VE]) {
-        const int h = (blockIdx.y * heads_per_wave + it) * 4 + wave;
-        if (it < heads_per_wave && h < heads && lane_on) VecLoad<T, VE>::load(qkv + ((size_t)n * heads + h) * D + e0, dst);
-        else {
-#pragma unroll
-            for (int i = 0; i < VE; ++i) dst[i] = 0.f;
-        }
+        const int h = min((blockIdx.y * heads_per_wave + it) * 4 + wave, heads - 1);
+        VecLoad<T, VE>::load(qkv + ((size_t)n * heads + h) * D + (lane_on ? e0 : 0), dst);
     };
     float v[VE], nxt[VE];
     load_head(0, v);
@@ -369,7 +367,10 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
         const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
         float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < VE; ++i) ss += v[i] * v[i];
+        for (int i = 0; i < VE; ++i) {
+            if (!lane_on) v[i] = 0.f;                       // lanes past the head size add nothing
+            ss += v[i] * v[i];
+        }
         const float* gain = is_q ? q_gain : (is_k ? k_gain : nullptr);
         if (gain && active) {
             ss = wave_sum(ss);
