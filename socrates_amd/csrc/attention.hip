@@ -762,7 +762,8 @@ __device__ __forceinline__ int pf_k_row(int k) {    // LDS row of key k of a til
     return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3);
 }
 
-template <int RT>
+// PAIR: pages hold an even, power-of-two number of keys, so a thread's two keys share a page.
+template <int RT, bool PAIR>
 __global__ void __launch_bounds__(256)
 paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                           const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -833,21 +834,35 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const bf16* k_base = k_pool + (size_t)kvh * BS * D + part_ld * 8;
     const bf16* v_base = v_pool + (size_t)kvh * BS * D + part_ld * 8;
     auto lookup = [&](int key0, int (&pg)[2]) {
+        if constexpr (PAIR) {
+            const int key = key0 + 2 * kp;
+            const bool ok = key + 1 >= kmin && key < khi;
+            pg[0] = pg[1] = table[ok ? key >> bs_shift : 0];
+        } else {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int key = key0 + 2 * kp + h;
-            const bool ok = key >= kmin && key < khi;
-            pg[h] = table[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
+            for (int h = 0; h < 2; ++h) {
+                const int key = key0 + 2 * kp + h;
+                const bool ok = key >= kmin && key < khi;
+                pg[h] = table[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
+            }
         }
     };
     auto fetch = [&](int key0, const int (&pg)[2], uint4 (&kr)[2], uint4 (&vr)[2]) {
+        if constexpr (PAIR) {
+            const size_t off = (size_t)pg[0] * page_stride + (size_t)(((key0 + 2 * kp) & (BS - 1)) * D);
+            kr[0] = *reinterpret_cast<const uint4*>(k_base + off);
+            kr[1] = *reinterpret_cast<const uint4*>(k_base + off + D);
+            vr[0] = *reinterpret_cast<const uint4*>(v_base + off);
+            vr[1] = *reinterpret_cast<const uint4*>(v_base + off + D);
+        } else {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int key = key0 + 2 * kp + h;
-            const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
-            const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
-            kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
-            vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
+            for (int h = 0; h < 2; ++h) {
+                const int key = key0 + 2 * kp + h;
+                const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
+                const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
+                kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
+                vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
+            }
         }
     };
     auto stash = [&](int buf, int key0, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
@@ -1040,10 +1055,15 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
     if constexpr (D <= 128) {
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2
-        if (row_tiles == 1)
-            hipLaunchKernelGGL(paged_attn_prefill_kernel<1>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+        const bool pair = bs_shift >= 1;
+        if (row_tiles == 1 && pair)
+            hipLaunchKernelGGL((paged_attn_prefill_kernel<1, true>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+        else if (row_tiles == 1)
+            hipLaunchKernelGGL((paged_attn_prefill_kernel<1, false>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+        else if (row_tiles == 2 && pair)
+            hipLaunchKernelGGL((paged_attn_prefill_kernel<2, true>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
         else if (row_tiles == 2)
-            hipLaunchKernelGGL(paged_attn_prefill_kernel<2>, dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
+            hipLaunchKernelGGL((paged_attn_prefill_kernel<2, false>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
         else
             return (int)hipErrorInvalidValue;
 #undef SOC_PF_ARGS
