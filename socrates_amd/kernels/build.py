@@ -41,7 +41,9 @@ MFMA_VGPR_MAX_HEAD = 128
 
 SOURCES = {"elementwise": "elementwise.hip", "gemm": "gemm.hip", "sampling": "sampling.hip",
            "attention": "attention.hip"}
-COMMON_HEAD_DIMS = (16, 32, 48, 64, 128)
+# head sizes built ahead by build_all(): the common ones and those the tests use, so that
+# no test compiles on the GPU box
+COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 112, 128, 256)
 
 _loaded = {}
 _lock = threading.Lock()
