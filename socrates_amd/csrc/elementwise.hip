@@ -420,6 +420,98 @@ qk_norm_rope_kernel(const T* __restrict__ qkv, T* __restrict__ q_out,
     }
 }
 
+// The same for many tokens, bfloat16, head sizes 64 and 128 and a rotation over the whole
+// head (or none): a lane owns eight consecutive elements (16-byte accesses), LPH = D / 8
+// lanes form a head and a wave works on 64 / LPH heads at once, which cuts the instructions
+// per head by that factor (the one-head-per-wave kernel is bound by them on long prompts).
+// Gains and the token's sines and cosines sit in registers; the sums cross lanes through DPP.
+template <int LPH>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_wide_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out, bf16* __restrict__ k_out,
+                         bf16* __restrict__ v_out, bf16* __restrict__ k_pool, bf16* __restrict__ v_pool,
+                         const int* __restrict__ block_table, int table_width,
+                         const int* __restrict__ token_rows, const int* __restrict__ positions,
+                         const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+                         const float* __restrict__ inv_freq, int Hq, int Hkv, int BS, float eps,
+                         int groups_per_wave) {
+    constexpr int D = LPH * 8, HPW = SOC_WAVE / LPH, half = D / 2;
+    __shared__ float cos_t[half], sin_t[half];
+    const int n = blockIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SOC_WAVE), lane = threadIdx.x % SOC_WAVE;
+    const int heads = Hq + 2 * Hkv;
+    const int sub = lane / LPH, e0 = (lane % LPH) * 8;
+    auto head_of = [&](int it) { return (((int)blockIdx.y * groups_per_wave + it) * 4 + wave) * HPW + sub; };
+    auto load_head = [&](int it) {                         // unconditional: a head outside reads the last one
+        return *reinterpret_cast<const uint4*>(qkv + ((size_t)n * heads + min(head_of(it), heads - 1)) * D + e0);
+    };
+    uint4 cur = load_head(0);
+    const int pos = positions ? positions[n] : 0;
+    float gq[8], gk[8], cs[8], sn[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { gq[i] = q_gain ? q_gain[e0 + i] : 1.f; gk[i] = k_gain ? k_gain[e0 + i] : 1.f; }
+    if (inv_freq) {
+        if ((int)threadIdx.x < half) sincosf((float)pos * inv_freq[threadIdx.x], &sin_t[threadIdx.x], &cos_t[threadIdx.x]);
+        __syncthreads();
+        const int j0 = e0 < half ? e0 : e0 - half;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { cs[i] = cos_t[j0 + i]; sn[i] = sin_t[j0 + i]; }
+    }
+    size_t page_base = 0;
+    if (k_pool) {
+        const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
+        page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;
+    }
+    for (int it = 0; it < groups_per_wave; ++it) {
+        const uint4 nxt = load_head(it + 1 < groups_per_wave ? it + 1 : it);
+        const int h = head_of(it);
+        const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
+        float v[8];
+        {
+            const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+        }
+        if ((is_q && q_gain) || (is_k && k_gain)) {         // the same for all lanes of a head
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+            ss += soc_dpp<SOC_DPP_XOR1>(ss);
+            ss += soc_dpp<SOC_DPP_XOR2>(ss);
+            ss += soc_dpp<SOC_DPP_HALF_MIRROR>(ss);
+            if constexpr (LPH == 16) ss += soc_dpp<SOC_DPP_ROW_MIRROR>(ss);
+            const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = v[i] * inv * (is_q ? gq[i] : gk[i]);
+        }
+        if (inv_freq) {
+            // the partner of element e is e +- D / 2: the same slot of the lane LPH / 2 away in the head
+            float partner[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if constexpr (LPH == 16) partner[i] = soc_dpp<0x128>(v[i]);          // rotate the row of 16 by 8
+                else partner[i] = __shfl_xor(v[i], LPH / 2, SOC_WAVE);
+            }
+            if (is_q || is_k) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    v[i] = e0 < half ? v[i] * cs[i] - partner[i] * sn[i] : v[i] * cs[i] + partner[i] * sn[i];
+            }
+        }
+        if (h < heads) {
+            bf16* dst;
+            if (is_q) dst = q_out + ((size_t)n * Hq + h) * D;
+            else {
+                const int kvh = is_k ? h - Hq : h - Hq - Hkv;
+                if (k_pool) dst = (is_k ? k_pool : v_pool) + page_base + (size_t)kvh * BS * D;
+                else dst = (is_k ? k_out : v_out) + ((size_t)n * Hkv + kvh) * D;
+            }
+            *reinterpret_cast<uint4*>(dst + e0) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
+                                                             pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
+        }
+        cur = nxt;
+    }
+}
+
 template <typename T>
 static void launch_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void* v_out, void* k_pool,
                                 void* v_pool, const int* block_table, int table_width,
@@ -427,6 +519,21 @@ static void launch_qk_norm_rope(const void* qkv, void* q_out, void* k_out, void*
                                 const float* k_gain, const float* inv_freq, int N, int Hq, int Hkv, int D,
                                 int rotary_dim, int BS, float eps, hipStream_t stream) {
     const int heads = Hq + 2 * Hkv;
+    if constexpr (sizeof(T) == 2) {
+        // many tokens, a head size and a rotation the wide kernel takes: several heads per wave
+        if (N >= 256 && (D == 64 || D == 128) && (!inv_freq || rotary_dim == D)) {
+            const int hpw_wide = D == 128 ? 4 : 8;
+            const int groups = (heads + hpw_wide - 1) / hpw_wide;
+            const int gpw = (groups + 3) / 4;
+            const dim3 grid_wide(N, 1);
+#define SOC_QKW_ARGS (const bf16*)qkv, (bf16*)q_out, (bf16*)k_out, (bf16*)v_out, (bf16*)k_pool, (bf16*)v_pool, \
+        block_table, table_width, token_rows, positions, q_gain, k_gain, inv_freq, Hq, Hkv, BS, eps, gpw
+            if (D == 128) hipLaunchKernelGGL(qk_norm_rope_wide_kernel<16>, grid_wide, dim3(256), 0, stream, SOC_QKW_ARGS);
+            else hipLaunchKernelGGL(qk_norm_rope_wide_kernel<8>, grid_wide, dim3(256), 0, stream, SOC_QKW_ARGS);
+#undef SOC_QKW_ARGS
+            return;
+        }
+    }
     // few tokens: one head per wave; many tokens: a workgroup walks all heads of its token
     const int hpw = N >= 256 ? (heads + 3) / 4 : 1;
     const dim3 grid(N, (heads + 4 * hpw - 1) / (4 * hpw));

@@ -375,6 +375,41 @@ def test_qk_norm_rope_write(kernel_sets, dtype, Hq, Hkv, D, rot):
     close(fresh.slot(0).k, caches[1].slot(0).k, dtype)
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,rope", [(32, 8, 128, True), (5, 1, 128, True), (6, 2, 64, True), (9, 3, 64, False),
+                                           (4, 2, 128, False)])
+def test_qk_norm_rope_write_long_prompts(kernel_sets, Hq, Hkv, D, rope):
+    """Hundreds of tokens in bfloat16 take the kernel that works on several heads per wave
+    (head sizes 64 and 128, rotation over the whole head or none); head counts that do not
+    fill the last wave, two rows, one of them continuing at position 37."""
+    from socrates_amd.cache import CacheManager
+    from socrates_amd.parts import PagedKV
+    dtype = torch.bfloat16
+    hip, ref = kernel_sets[dtype]
+    bs = 16
+    caches = [CacheManager([PagedKV(Hkv, D)], 2, 512, bs, 40, dtype, DEV) for _ in range(2)]
+    for c in caches:
+        r0, r1 = c.open_row(), c.open_row()
+        c.reserve(r0, 200)
+        c.reserve(r1, 37)
+        c.advance(r1, 37)
+        c.reserve(r1, 37 + 131)
+        c.sync()
+    rows = [0] * 200 + [1] * 131
+    pos = list(range(200)) + list(range(37, 37 + 131))
+    N = len(rows)
+    positions = torch.tensor(pos, dtype=torch.int32, device=DEV)
+    token_rows = torch.tensor(rows, dtype=torch.int32, device=DEV)
+    qkv = rnd((N, (Hq + 2 * Hkv) * D), dtype, 31)
+    qg, kg = (1 + 0.2 * torch.randn(D)).to(DEV), (1 + 0.2 * torch.randn(D)).to(DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, D, 2).float() / D))).to(DEV) if rope else None
+    args = (qkv, Hq, Hkv, D, qg, kg, 1e-6, inv_freq, D if rope else 0, positions, token_rows)
+    got = hip.qk_norm_rope_write(*args, caches[0].slot(0))
+    want = ref.qk_norm_rope_write(*args, caches[1].slot(0))
+    close(got, want, dtype)
+    close(caches[0].slot(0).k, caches[1].slot(0).k, dtype)
+    close(caches[0].slot(0).v, caches[1].slot(0).v, dtype, atol=0, rtol=0)
+
+
 def test_rope_properties(kernel_sets):
     """Position 0 is the identity; pair norms are kept; <rope(q, m), rope(k, n)> depends on
     m - n only; equals complex multiplication by e^{i pos theta^(-2j/D)}."""
