@@ -395,11 +395,13 @@ class HipKernels:
                 raise KernelError("more than 65535 tokens in one attention call")
             wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2) else (2 if D <= 64 else 1)
             wg_tokens = 4 * max(1, (16 * wg_rt) >> gpl)
-            # Prompt portions go to the kernel whose four waves share the K and V tiles, if its
-            # workgroups fill the GPU (it has no key splits); a short portion behind a long
-            # context is better served by the per-wave kernel with key splits. An override of
+            # Prompt portions go to the kernel whose four waves share the K and V tiles, if it
+            # has a workgroup for every compute unit (it has no key splits; measured: 512
+            # tokens behind 3.5 k of context, 256 workgroups, 107 us against 187 us); a
+            # shorter portion behind a long context is better served by the per-wave kernel
+            # with key splits (128 tokens behind 8 k: 95 us against 196 us). An override of
             # the row tiles (tests) forces the choice.
-            enough = (N // wg_tokens) * Hkv * ((G + 15) // 16) >= 512 or self.attention_row_tiles is not None
+            enough = (N // wg_tokens) * Hkv * ((G + 15) // 16) >= 256 or self.attention_row_tiles is not None
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt
