@@ -370,7 +370,8 @@ class HipKernels:
             split_len = max(16, (min(split_len, 1 << 24) + 15) // 16 * 16)
             return split_len, max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
         waves = n_blocks * n_kv_heads * ((group + 15) // 16)
-        n = max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64))
+        # from one wave per SIMD on (1,024) no split: the merge costs a wave per (token, head)
+        n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64))
         split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
         return split_len, (max_keys + split_len - 1) // split_len
 
