@@ -541,15 +541,15 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         fetch(key0 + 80, pg2, kf2, vr2);
         pg2 = lookup(key0 + 128);
     }
-    tile(key0, kf0, vr0);
-    if (key0 + 48 < khi) fetch(key0 + 48, pg0, kf0, vr0);
-    if (key0 + 16 < khi) {
+    for (; key0 < khi; key0 += 48) {                         // at most two rounds: five tiles
+        tile(key0, kf0, vr0);
+        if (key0 + 48 < khi) fetch(key0 + 48, pg0, kf0, vr0);
+        if (key0 + 16 >= khi) break;
         tile(key0 + 16, kf1, vr1);
         if (key0 + 64 < khi) fetch(key0 + 64, pg1, kf1, vr1);
+        if (key0 + 32 >= khi) break;
+        tile(key0 + 32, kf2, vr2);
     }
-    if (key0 + 32 < khi) tile(key0 + 32, kf2, vr2);
-    if (key0 + 48 < khi) tile(key0 + 48, kf0, vr0);
-    if (key0 + 64 < khi) tile(key0 + 64, kf1, vr1);
 
     // finish: the row sum is spread over the four lanes of the row's column
 #pragma unroll
