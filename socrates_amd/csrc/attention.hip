@@ -762,8 +762,17 @@ __device__ __forceinline__ int pf_k_row(int k) {    // LDS row of key k of a til
     return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3);
 }
 
+// LDS row of key k of a tile for the 32-row products: bits 2 and 3 of k change places, so that
+// the 16 scores a lane gets from one 32 x 32 product are two runs of eight neighbouring keys,
+// which is what the second product wants from it as operand B.
+__device__ __forceinline__ int pf_k_row32(int k) { return (k & ~12) | ((k & 4) << 1) | ((k & 8) >> 1); }
+
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
 // PAIR: pages hold an even, power-of-two number of keys, so a thread's two keys share a page.
-template <int RT, bool PAIR>
+// M32: a wave owns 32 rows and multiplies with the 32 x 32 x 16 instruction (RT = 1; head
+// sizes that are multiples of 32): per row, half the loads, LDS reads, stores and barriers.
+template <int RT, bool PAIR, bool M32>
 __global__ void __launch_bounds__(256)
 paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                           const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -784,7 +793,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int tok0 = row_blocks ? row_blocks[2 * blk] : blk, ntok = row_blocks ? row_blocks[2 * blk + 1] : 1;
     const int pos0 = positions[tok0];
     const int* table = block_table + (size_t)token_rows[tok0] * table_width;
-    const int tokens_per_wave = (16 * RT) >> group_pad_log2;
+    const int tokens_per_wave = ((M32 ? 32 : 16 * RT)) >> group_pad_log2;
 
     const int khi = pos0 + ntok;                                    // keys any row of the block sees
     const int kmin = window > 0 ? max(0, pos0 - window + 1) : 0;
@@ -817,6 +826,32 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         m[rt] = -INFINITY; l[rt] = 0.f;
 #pragma unroll
         for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    }
+    // 32-row products: the lane's row is lane % 32, its half of every 16-wide k step lane / 32
+    constexpr int DQ32 = D / 16, DB32 = D / 32;
+    const int c32 = lane % 32, g32 = lane / 32;
+    int row_pos32 = -1;
+    size_t row_q32 = 0;
+    // the lane's slices of its query row wait in LDS (each lane reads back what it wrote):
+    // with them in registers a wave would need more than half of a SIMD's registers
+    __shared__ __align__(16) uint16_t q_lds[M32 ? 4 * 32 * PF_K_STRIDE : 8];
+    const int q_off = M32 ? (wave * 32 + c32) * PF_K_STRIDE + 8 * g32 : 0;
+    uint16_t* q_mine = q_lds + q_off;
+    f32x16_t o32[M32 ? DB32 : 1];
+    float m32 = -INFINITY, l32 = 0.f;
+    if constexpr (M32) {
+        const int tt = wtok0 + (c32 >> group_pad_log2), gh = chunk * 16 + (c32 & (Gp - 1));
+        const bool ok = tt < ntok && gh < G;
+        row_pos32 = ok ? pos0 + tt : -1;
+        row_q32 = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? gh : 0)) * D;
+#pragma unroll
+        for (int t = 0; t < DQ32; ++t)
+            *reinterpret_cast<uint4*>(q_mine + 16 * t) =
+                ok ? *reinterpret_cast<const uint4*>(q + row_q32 + 16 * t + 8 * g32) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+        for (int b = 0; b < DB32; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o32[b][i] = 0.f;
     }
 
     // Cooperative tile loads: a thread owns two neighbouring keys (2 kp, 2 kp + 1) and one
@@ -873,8 +908,9 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             if (key < kmin || key >= khi) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
             if (key + 1 < kmin || key + 1 >= khi) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
         }
-        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp) * PF_K_STRIDE + part * 8]) = k0;
-        *reinterpret_cast<uint4*>(&k_lds[buf][pf_k_row(2 * kp + 1) * PF_K_STRIDE + part * 8]) = k1;
+        const int r0 = M32 ? pf_k_row32(2 * kp) : pf_k_row(2 * kp), r1 = M32 ? pf_k_row32(2 * kp + 1) : pf_k_row(2 * kp + 1);
+        *reinterpret_cast<uint4*>(&k_lds[buf][r0 * PF_K_STRIDE + part * 8]) = k0;
+        *reinterpret_cast<uint4*>(&k_lds[buf][r1 * PF_K_STRIDE + part * 8]) = k1;
         const uint32_t a[4] = {v0.x, v0.y, v0.z, v0.w};
         const uint32_t b[4] = {v1.x, v1.y, v1.z, v1.w};
         uint32_t* vt = reinterpret_cast<uint32_t*>(&v_lds[buf][(part * 8) * PF_V_STRIDE + 2 * kp]);
@@ -961,6 +997,74 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                     o[rt][j], 0, 0, 0);
     };
 
+    // The same with 32 rows per wave: S^T [32 keys x 32 rows] from D / 16 products, a row's
+    // scores in two lanes (16 each), O^T [32 d x 32 rows] per 32-wide block of d.
+    auto compute32 = [&](int key0, int buf, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const uint16_t* kt = k_lds[buf];
+        const uint16_t* vt = v_lds[buf];
+        f32x16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+        int q_at = q_off;
+        asm volatile("" : "+v"(q_at));                      // read every tile anew: not hoisted back into registers
+        const uint16_t* q_mine = q_lds + q_at;
+#pragma unroll
+        for (int t = 0; t < DQ32; ++t) {
+            const uint4 ka = *reinterpret_cast<const uint4*>(kt + c32 * PF_K_STRIDE + 16 * t + 8 * g32);
+            const uint4 qa = *reinterpret_cast<const uint4*>(q_mine + 16 * t);
+            sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t*>(&ka),
+                                                         *reinterpret_cast<const bf16x8_t*>(&qa), sc, 0, 0, 0);
+        }
+        float tv[16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            tv[i] = sc[i] * c2;
+            if constexpr (MASKED) {
+                const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
+                bool seen = key <= row_pos32;
+                if (window > 0) seen = seen && key > row_pos32 - window;
+                tv[i] = seen ? tv[i] : -INFINITY;
+            }
+            mx = fmaxf(mx, tv[i]);
+        }
+        mx = max_xor32(mx);
+        const float mn = fmaxf(m32, mx);
+        const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
+        const float alpha = __builtin_amdgcn_exp2f(m32 - ms);
+        float p[16];
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(tv[i] - ms);
+            psum += p[i];
+        }
+        l32 = l32 * alpha + psum;
+        const bool rescale = m32 != mn;
+        m32 = mn;
+        uint4 pf[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            pf[h] = make_uint4(pack_bf16x2(p[8 * h], p[8 * h + 1]), pack_bf16x2(p[8 * h + 2], p[8 * h + 3]),
+                               pack_bf16x2(p[8 * h + 4], p[8 * h + 5]), pack_bf16x2(p[8 * h + 6], p[8 * h + 7]));
+        if (__any(rescale)) {
+#pragma unroll
+            for (int b = 0; b < DB32; ++b) o32[b] *= alpha;
+        }
+#pragma unroll
+        for (int b = 0; b < DB32; ++b) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint2* src = reinterpret_cast<const uint2*>(vt + (32 * b + c32) * PF_V_STRIDE + 16 * h + 8 * g32);
+                const uint2 lo = src[0], hi = src[1];
+                const uint4 va = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                o32[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t*>(&va),
+                                                                  *reinterpret_cast<const bf16x8_t*>(&pf[h]), o32[b], 0, 0, 0);
+            }
+        }
+    };
+
     // Two tiles of global loads are in flight while one is computed: at the top of the
     // iteration of tile t, tile t sits in LDS buffer t % 2, the loads of tile t + 1 are on
     // their way into one pair of staging registers, and the pages of tile t + 2 were asked
@@ -977,8 +1081,13 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             // the window of its last one
             const bool whole = key0 + PF_KEYS - 1 <= wave_lo_pos &&
                                (window <= 0 || key0 > wave_hi_pos - window);
-            if (whole) compute(key0, buf, std::false_type{});
-            else compute(key0, buf, std::true_type{});
+            if constexpr (M32) {
+                if (whole) compute32(key0, buf, std::false_type{});
+                else compute32(key0, buf, std::true_type{});
+            } else {
+                if (whole) compute(key0, buf, std::false_type{});
+                else compute(key0, buf, std::true_type{});
+            }
         }
     };
     int pg0[2], pg1[2];
@@ -1017,6 +1126,22 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         }
     }
 
+    if constexpr (M32) {
+        const float L = sum_xor32(l32);
+        if (row_pos32 >= 0) {
+            const float inv = L > 0.f ? 1.0f / L : 0.f;
+#pragma unroll
+            for (int b = 0; b < DB32; ++b)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {                 // o32[b][4a + j] is d = 32 b + 8 a + 4 g32 + j
+                    uint2 pk;
+                    pk.x = pack_bf16x2(o32[b][4 * a] * inv, o32[b][4 * a + 1] * inv);
+                    pk.y = pack_bf16x2(o32[b][4 * a + 2] * inv, o32[b][4 * a + 3] * inv);
+                    *reinterpret_cast<uint2*>(out + row_q32 + 32 * b + 8 * a + 4 * g32) = pk;
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         float L = l[rt];
@@ -1035,7 +1160,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 
 // bfloat16 only, head sizes up to 128, no key splits. row_blocks [n_row_blocks, 2] = (first
 // token, tokens) of each block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of
-// one sequence, or null: every token is a block of its own.
+// one sequence, or null: every token is a block of its own. row_tiles 32: a wave owns 32 rows
+// (blocks of at most 4 * (32 >> group_pad_log2) tokens), head sizes that are multiples of 32.
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
@@ -1056,16 +1182,18 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2
         const bool pair = bs_shift >= 1;
-        if (row_tiles == 1 && pair)
-            hipLaunchKernelGGL((paged_attn_prefill_kernel<1, true>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-        else if (row_tiles == 1)
-            hipLaunchKernelGGL((paged_attn_prefill_kernel<1, false>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-        else if (row_tiles == 2 && pair)
-            hipLaunchKernelGGL((paged_attn_prefill_kernel<2, true>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-        else if (row_tiles == 2)
-            hipLaunchKernelGGL((paged_attn_prefill_kernel<2, false>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);
-        else
-            return (int)hipErrorInvalidValue;
+#define SOC_PF_LAUNCH(RT_, M32_)                                                                            \
+    do {                                                                                                    \
+        if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS); \
+        else hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, false, M32_>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);     \
+    } while (0)
+        if (row_tiles == 1) SOC_PF_LAUNCH(1, false);
+        else if (row_tiles == 2) SOC_PF_LAUNCH(2, false);
+        else if (row_tiles == 32) {                          // 32 rows per wave through the 32 x 32 products
+            if constexpr (D % 32 == 0) SOC_PF_LAUNCH(1, true);
+            else return (int)hipErrorInvalidValue;
+        } else return (int)hipErrorInvalidValue;
+#undef SOC_PF_LAUNCH
 #undef SOC_PF_ARGS
         return soc_last_error();
     } else {

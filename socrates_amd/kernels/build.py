@@ -43,7 +43,7 @@ SOURCES = {"elementwise": "elementwise.hip", "gemm": "gemm.hip", "sampling": "sa
            "attention": "attention.hip"}
 # head sizes built ahead by build_all(): the common ones and those the tests use, so that
 # no test compiles on the GPU box
-COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 112, 128, 256)
+COMMON_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 256)
 
 _loaded = {}
 _lock = threading.Lock()
