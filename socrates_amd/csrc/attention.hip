@@ -772,8 +772,13 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 // PAIR: pages hold an even, power-of-two number of keys, so a thread's two keys share a page.
 // M32: a wave owns 32 rows and multiplies with the 32 x 32 x 16 instruction (RT = 1; head
 // sizes that are multiples of 32): per row, half the loads, LDS reads, stores and barriers.
-template <int RT, bool PAIR, bool M32>
-__global__ void __launch_bounds__(256)
+// KS = 2 (with M32): eight waves; waves 0-3 walk the first half of the block's key tiles and
+// waves 4-7, with the same rows, the second half, each four with tiles of their own in LDS;
+// at the end the two partial results are combined through LDS. Twice the waves for the same
+// number of workgroups: for launches whose workgroups are too few, or too uneven (a prompt
+// from its start: the last block sees all keys, the first none), to fill the GPU otherwise.
+template <int RT, bool PAIR, bool M32, int KS>
+__global__ void __launch_bounds__(256 * KS)
 paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                           const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
                           int table_width, const int* __restrict__ token_rows,
@@ -781,9 +786,14 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                           bf16* __restrict__ out, int Hq, int Hkv, int BS, int bs_shift, float scale,
                           int window, int group_pad_log2) {
     static_assert(D <= 128, "one key pair per thread");
-    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][PF_K_ELEMS];
-    __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][PF_V_ELEMS];
-    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
+    static_assert(KS == 1 || (KS == 2 && M32), "key halves come with the 32-row products");
+    constexpr int PF_TILE_ELEMS = PF_K_ELEMS + PF_V_ELEMS;          // one K tile and one V^T tile
+    __shared__ __attribute__((aligned(16))) uint16_t tiles_lds[KS * 2 * PF_TILE_ELEMS];
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x / SOC_WAVE), lane = threadIdx.x % SOC_WAVE;
+    const int half = wave_all / 4, wave = wave_all % 4;             // which keys, which rows
+    const int tid = threadIdx.x % 256;                              // among the four waves that share tiles
+    uint16_t* const k_lds[2] = {tiles_lds + (half * 2) * PF_TILE_ELEMS, tiles_lds + (half * 2 + 1) * PF_TILE_ELEMS};
+    uint16_t* const v_lds[2] = {k_lds[0] + PF_K_ELEMS, k_lds[1] + PF_K_ELEMS};
     const int li = lane % 16, kb = lane / 16;
     const int G = Hq / Hkv, Gp = 1 << group_pad_log2;
     const int chunks = (G + 15) / 16;
@@ -797,7 +807,16 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 
     const int khi = pos0 + ntok;                                    // keys any row of the block sees
     const int kmin = window > 0 ? max(0, pos0 - window + 1) : 0;
-    const int klo = kmin & ~(PF_KEYS - 1);
+    int klo = kmin & ~(PF_KEYS - 1);
+    // kend: where this half's walk over the tiles ends. Both halves take the same number of
+    // steps (they share the barriers); the second may run past khi, where keys are stand-ins
+    // that no row sees.
+    int kend = khi;
+    if constexpr (KS == 2) {
+        const int per_half = ((khi - klo + PF_KEYS - 1) / PF_KEYS + 1) / 2 * PF_KEYS;
+        klo += half * per_half;
+        kend = klo + per_half;
+    }
     // this wave's rows
     const int wtok0 = wave * tokens_per_wave;                       // first token of the wave in the block
     const int wave_lo_pos = pos0 + wtok0;                           // its first and last positions
@@ -834,8 +853,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     size_t row_q32 = 0;
     // the lane's slices of its query row wait in LDS (each lane reads back what it wrote):
     // with them in registers a wave would need more than half of a SIMD's registers
-    __shared__ __align__(16) uint16_t q_lds[M32 ? 4 * 32 * PF_K_STRIDE : 8];
-    const int q_off = M32 ? (wave * 32 + c32) * PF_K_STRIDE + 8 * g32 : 0;
+    __shared__ __align__(16) uint16_t q_lds[M32 ? KS * 4 * 32 * PF_K_STRIDE : 8];
+    const int q_off = M32 ? (wave_all * 32 + c32) * PF_K_STRIDE + 8 * g32 : 0;
     uint16_t* q_mine = q_lds + q_off;
     f32x16_t o32[M32 ? DB32 : 1];
     float m32 = -INFINITY, l32 = 0.f;
@@ -1096,11 +1115,11 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     lookup(klo + PF_KEYS, pg1);
     fetch(klo, pg0, kr0, vr0);
     lookup(klo + 2 * PF_KEYS, pg0);
-    if (klo + PF_KEYS < khi) fetch(klo + PF_KEYS, pg1, kr1, vr1);
+    if (klo + PF_KEYS < kend) fetch(klo + PF_KEYS, pg1, kr1, vr1);
     stash(0, klo, kr0, vr0);
     __syncthreads();
     int key0 = klo;
-    for (; key0 + 3 * PF_KEYS < khi; key0 += 2 * PF_KEYS) {
+    for (; key0 + 3 * PF_KEYS < kend; key0 += 2 * PF_KEYS) {
         lookup(key0 + 3 * PF_KEYS, pg1);
         fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
         tile(key0, 0);
@@ -1112,7 +1131,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         stash(0, key0 + 2 * PF_KEYS, kr0, vr0);
         __syncthreads();
     }
-    const bool has1 = key0 + PF_KEYS < khi, has2 = key0 + 2 * PF_KEYS < khi;      // the same in all threads
+    const bool has1 = key0 + PF_KEYS < kend, has2 = key0 + 2 * PF_KEYS < kend;    // the same in all threads
     if (has2) fetch(key0 + 2 * PF_KEYS, pg0, kr0, vr0);
     tile(key0, 0);
     if (has1) {
@@ -1127,7 +1146,32 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     }
 
     if constexpr (M32) {
-        const float L = sum_xor32(l32);
+        float L = sum_xor32(l32);
+        if constexpr (KS == 2) {
+            // the second half hands its result over: [wave][value][lane] floats where the tiles were
+            static_assert(KS * 2 * PF_TILE_ELEMS * 2 >= 4 * 64 * (16 * DB32 + 2) * 4, "the tiles' space holds the exchange");
+            float* xch = reinterpret_cast<float*>(tiles_lds) + (size_t)wave * (16 * DB32 + 2) * 64 + lane;
+            __syncthreads();                                 // every wave is done with the tiles
+            if (half == 1) {
+#pragma unroll
+                for (int b = 0; b < DB32; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) xch[(16 * b + i) * 64] = o32[b][i];
+                xch[(16 * DB32) * 64] = m32;
+                xch[(16 * DB32 + 1) * 64] = L;
+            }
+            __syncthreads();
+            if (half == 1) return;
+            const float m_b = xch[(16 * DB32) * 64], l_b = xch[(16 * DB32 + 1) * 64];
+            const float mn = fmaxf(m32, m_b);
+            const float ms = mn == -INFINITY ? 0.f : mn;
+            const float wa = __builtin_amdgcn_exp2f(m32 - ms), wb = __builtin_amdgcn_exp2f(m_b - ms);
+            L = L * wa + l_b * wb;
+#pragma unroll
+            for (int b = 0; b < DB32; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o32[b][i] = o32[b][i] * wa + xch[(16 * b + i) * 64] * wb;
+        }
         if (row_pos32 >= 0) {
             const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll
@@ -1161,7 +1205,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 // bfloat16 only, head sizes up to 128, no key splits. row_blocks [n_row_blocks, 2] = (first
 // token, tokens) of each block of at most 4 * ((16 * row_tiles) >> group_pad_log2) tokens of
 // one sequence, or null: every token is a block of its own. row_tiles 32: a wave owns 32 rows
-// (blocks of at most 4 * (32 >> group_pad_log2) tokens), head sizes that are multiples of 32.
+// (blocks of at most 4 * (32 >> group_pad_log2) tokens), head sizes that are multiples of 32;
+// row_tiles 64: the same with eight waves, four for each half of a block's keys.
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
@@ -1182,16 +1227,18 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2
         const bool pair = bs_shift >= 1;
-#define SOC_PF_LAUNCH(RT_, M32_)                                                                            \
+#define SOC_PF_LAUNCH(RT_, M32_, KS_)                                                                            \
     do {                                                                                                    \
-        if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS); \
-        else hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, false, M32_>), dim3((unsigned)groups), dim3(256), 0, stream, SOC_PF_ARGS);     \
+        if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_, KS_>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS); \
+        else hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, false, M32_, KS_>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS);     \
     } while (0)
-        if (row_tiles == 1) SOC_PF_LAUNCH(1, false);
-        else if (row_tiles == 2) SOC_PF_LAUNCH(2, false);
-        else if (row_tiles == 32) {                          // 32 rows per wave through the 32 x 32 products
-            if constexpr (D % 32 == 0) SOC_PF_LAUNCH(1, true);
-            else return (int)hipErrorInvalidValue;
+        if (row_tiles == 1) SOC_PF_LAUNCH(1, false, 1);
+        else if (row_tiles == 2) SOC_PF_LAUNCH(2, false, 1);
+        else if (row_tiles == 32 || row_tiles == 64) {       // 32 rows per wave through the 32 x 32 products
+            if constexpr (D % 32 == 0) {
+                if (row_tiles == 32) SOC_PF_LAUNCH(1, true, 1);
+                else SOC_PF_LAUNCH(1, true, 2);              // and the keys of a block in two halves
+            } else return (int)hipErrorInvalidValue;
         } else return (int)hipErrorInvalidValue;
 #undef SOC_PF_LAUNCH
 #undef SOC_PF_ARGS

@@ -85,6 +85,7 @@ class HipKernels:
         _declare(self._sampling, _SAMPLING_SIGNATURES)
         self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
         self.attention_row_tiles = None     # row tiles per wave of the MFMA kernel, override
+        self.last_attention_kernel = None   # (kernel, row tiles) the last bfloat16 call went to
         self.attention_mfma = True          # bfloat16 takes the MFMA kernels
         self.attention_workgroup = True     # prompt portions take the kernel that shares K/V through LDS
         # bfloat16 products with more than 16 rows go to the library (hipBLASLt through
@@ -395,19 +396,25 @@ class HipKernels:
             if N > 65535:
                 raise KernelError("more than 65535 tokens in one attention call")
             # row tiles 32: 32 rows per wave through the 32 x 32 products (head sizes in steps of 32)
-            wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2, 32) else (2 if D <= 64 else 1)
-            if wg_rt == 32 and D % 32:
+            # 64: the same with eight waves, each four on one half of a block's keys
+            wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2, 32, 64) else (2 if D <= 64 else 1)
+            if wg_rt >= 32 and D % 32:
                 wg_rt = 1
             if self.attention_row_tiles is None and D > 64 and D % 32 == 0:
                 # head sizes 96 and 128 (64 and less hold two row tiles anyway): 20 % faster
                 # where its workgroups, half as many, still fill the GPU evenly: two for every
                 # slot (512 of four waves), or one if no row sees less than half the keys of
-                # another. Measured at 8 kv heads of 4 x 128: 2,048 tokens behind 6,144:
-                # 370 us against 442 us; 4,096 from 0: 231 against 273; 2,048 from 0: the same.
+                # another. Uneven and one per slot (a prompt of 2,048 tokens from its start):
+                # the eight-wave form, which splits each block's keys inside the workgroup.
+                # Measured at 8 kv heads of 4 x 128, 16 / 32 / 32 rows in two halves:
+                # 2,048 tokens behind 6,144: 436 / 355 / 376 us; 4,096 from 0: 267 / 222 / 241;
+                # 2,048 from 0: 91 / 88 / 78; 1,024 from 0: 34 / 43 / 36.
                 n32 = (N // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16)
                 if n32 >= 1024 or (n32 >= 512 and ctx.max_ctx_len >= 2 * getattr(ctx, "max_q_len", 1)):
                     wg_rt = 32
-            wg_tokens = 4 * max(1, (32 if wg_rt == 32 else 16 * wg_rt) >> gpl)
+                elif n32 >= 512:
+                    wg_rt = 64
+            wg_tokens = 4 * max(1, (32 if wg_rt >= 32 else 16 * wg_rt) >> gpl)
             # Prompt portions go to the kernel whose four waves share the K and V tiles, if it
             # has a workgroup for every compute unit (it has no key splits; measured: 512
             # tokens behind 3.5 k of context, 256 workgroups, 107 us against 187 us); a
@@ -418,6 +425,7 @@ class HipKernels:
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt
+                self.last_attention_kernel = ("workgroup", rt)
                 blocks, n_blocks = self._row_blocks(ctx, N, wg_tokens)
                 _check(lib.soc_paged_attention_prefill(
                     _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
@@ -429,6 +437,7 @@ class HipKernels:
             rt = self.attention_row_tiles or 1
             rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
             tokens_per_block = max(1, (16 * rt) >> gpl)
+            self.last_attention_kernel = ("wave", rt)
             blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
             split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
             part_o = part_ml = None

@@ -244,7 +244,7 @@ def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     for window in (None, 1, 7, 16, 64):
         want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
         # (row tiles, splits, workgroup kernel): the per-wave and the workgroup MFMA kernels
-        for row_tiles, splits, wg in ((None, None, True), (1, None, True), (2, None, True), (32, None, True), (1, (32, 5), False),
+        for row_tiles, splits, wg in ((None, None, True), (1, None, True), (2, None, True), (32, None, True), (64, None, True), (1, (32, 5), False),
                                       (2, None, False), (4, (64, 3), False), (4, None, False)):
             hip.attention_row_tiles, hip.attention_splits, hip.attention_workgroup = row_tiles, splits, wg
             got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
@@ -268,33 +268,29 @@ def test_prefill_attention_whole_prompts(kernel_sets, Hq, Hkv, D, bs):
     q = rnd((len(rows), Hq, D), torch.bfloat16, 21)
     for window in (None, 40, 97):
         want = dense_attention(q, dense, rows, pos, D ** -0.5, window)
-        for rt in (1, 2, 32):                               # 32: the 32 x 32 products, head sizes in steps of 32
+        for rt in (1, 2, 32, 64):        # 32: the 32 x 32 products (head sizes in steps of 32); 64: keys in two halves
             hip.attention_row_tiles = rt
             got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5, window)
             close(got.cpu(), want, torch.bfloat16)
     hip.attention_row_tiles = None
 
 
-def test_prefill_attention_long_portion_behind_a_context(kernel_sets):
-    """A portion long enough that head size 128 goes to the 32-row products by itself
-    (512 workgroups of 8 tokens x 16 heads of a group, every row sees at least half the keys
-    that the last one sees); one key far back made to stand out for one query."""
+@pytest.mark.parametrize("start,row_tiles", [(1024, 32), (0, 64)])
+def test_prefill_attention_long_portions_choose_the_32_row_products(kernel_sets, start, row_tiles):
+    """Portions long enough that head size 128 goes to the 32-row products by itself (512
+    workgroups of 8 tokens x 16 heads of a group): behind a context, where every row sees at
+    least half the keys that the last one sees, with four waves; from the start of a prompt
+    with eight, each four on half of the keys. One early key is made to stand out for one query."""
     hip, _ = kernel_sets[torch.bfloat16]
     Hq, Hkv, D, bs = 64, 4, 128, 16
-    start, T = 1024, 1024
+    T = 1024
     slot, dense = make_paged_case([start + T], Hq, Hkv, D, bs, torch.bfloat16, seed=5)
     rows, pos = [0] * T, list(range(start, start + T))
     q = rnd((T, Hq, D), torch.bfloat16, 22)
     k0, v0 = dense[0]
     q[700, 37] = (8.0 * k0[37 // 16, 3]).to(torch.bfloat16)         # query 700 of head 37 looks at key 3
-    asked = []
-    plain_row_blocks = hip._row_blocks
-    hip._row_blocks = lambda ctx, n, per: asked.append(per) or plain_row_blocks(ctx, n, per)
-    try:
-        got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5)
-    finally:
-        hip._row_blocks = plain_row_blocks
-    assert asked == [8]                                                # 4 waves x (32 rows / 16 heads)
+    got = hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5)
+    assert hip.last_attention_kernel == ("workgroup", row_tiles)
     want = dense_attention(q, dense, rows, pos, D ** -0.5)
     close(got.cpu(), want, torch.bfloat16)
     assert (got[700].view(Hq, D)[37].float().cpu() - v0[37 // 16, 3]).abs().max() < 0.05
