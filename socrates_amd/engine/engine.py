@@ -151,6 +151,32 @@ class Engine:
             if self.step() == 0 and not self.scheduler.idle:
                 raise RuntimeError("requests are waiting but nothing can be scheduled")
 
+    def tune(self, token_counts: Optional[Sequence[int]] = None) -> None:
+        """Before serving: run a throwaway prompt of each of these lengths with the library
+        timing its solutions for the model's products at that many rows (about a second per
+        shape), and keep the fastest. Default: a full portion, and the largest batch if the
+        library serves it (more than 16 rows). Steps with other numbers of rows are not
+        affected. Decode graphs are captured afterwards, so they replay the kept choices."""
+        if not self.scheduler.idle:
+            raise RuntimeError("tune() runs on an idle engine")
+        ops = self.runner.ops
+        if not hasattr(ops, "library_tuning"):
+            return
+        if token_counts is None:
+            token_counts = [self.scheduler.token_budget] + ([self.max_batch] if self.max_batch > 16 else [])
+        kept = (self.n_steps, self.prompt_tokens, self.output_tokens)
+        ops.library_tuning(True)
+        try:
+            for n in token_counts:
+                n = max(1, min(int(n), self.scheduler.token_budget, self.max_len - 1))
+                self.submit([i % self.plan_.vocab_size for i in range(n)],
+                            sampling=SamplingParams(max_new_tokens=1, eos_token_ids=()))
+                self.run()
+                self.scheduler.retire_finished()
+        finally:
+            ops.library_tuning(False)
+        self.n_steps, self.prompt_tokens, self.output_tokens = kept
+
     # -- the Python entry point ------------------------------------------------------------------
     def generate(self, prompts: Sequence, max_new_tokens: Optional[int] = None,
                  temperature: float = 0.0, seed: int = 0,

@@ -200,6 +200,22 @@ class HipKernels:
         return self.swiglu(self.linear(x, w_gate_up), interleave)
 
     # -- matrix products ------------------------------------------------------------------------
+    def library_tuning(self, on: bool) -> None:
+        """While on, the library's matrix products (bfloat16, more than 16 rows) time the
+        library's solutions for every new shape they meet and keep the fastest; afterwards
+        the kept choices stay in use, for this process, and shapes met later take the
+        library's default. The library's record of its choices goes to a file of this
+        process in the temporary folder, never to the working folder."""
+        import os
+        import tempfile
+        import torch.cuda.tunable as tunable
+        if on:
+            tunable.set_filename(os.path.join(tempfile.gettempdir(), f"socrates_amd_products_{os.getpid()}.csv"))
+            tunable.enable(True)
+            tunable.set_max_tuning_duration(30)          # ms per solution
+            tunable.set_max_tuning_iterations(20)
+        tunable.tuning_enable(bool(on))
+
     def linear(self, x, w, out_dtype=None, allow_partial=False, row_tiles=0, n_waves=0, k_splits=0):
         """x [M, K] times w [N, K] transposed. float32 operands (either) take the plain
         float32 kernel. bfloat16 pairs: up to 16 rows the skinny MFMA kernel (it streams

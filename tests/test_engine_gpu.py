@@ -71,6 +71,32 @@ def test_temperature_tiny_b_workload(tmp_path):
             ids.append(tok)
 
 
+def test_tuned_library_products_leave_the_tokens_alone(tmp_path):
+    """``Engine.tune``: the library picks its fastest solution for the products of a 33-token
+    portion (bfloat16, more than 16 rows); greedy tokens stay those of the plain run, the
+    counters and the cache are as before, and nothing is written to the working folder."""
+    import os
+    from socrates_amd.engine import Engine
+    folder = write_tiny(tmp_path / "A", TINY_A, seed=0)
+    cfg, w = plain.read_folder(folder, torch.float64)
+    prompts = random_prompts([33, 20], cfg["vocab_size"], seed=3)
+    want = [plain.greedy(cfg, w, p, 6) for p in prompts]
+    engine = Engine(str(folder), dtype=torch.bfloat16, max_batch=4, max_len=64, max_new_tokens=6, block_size=16)
+    before = set(os.listdir("."))
+    engine.tune([33, 20])
+    assert (engine.n_steps, engine.prompt_tokens, engine.output_tokens) == (0, 0, 0)
+    assert engine.cache.n_free_pages == 4 * 4 and not engine.cache.open_rows
+    got = engine.generate(prompts)
+    for p, g, x in zip(prompts, got, want):
+        if margins_ok(cfg, w, p, x, 0.05):
+            assert g == x
+    with pytest.raises(RuntimeError):
+        engine.submit(prompts[0])
+        engine.tune()
+    engine.run()
+    assert set(os.listdir(".")) == before
+
+
 def test_command_line(tmp_path):
     folder = write_tiny(tmp_path / "A", TINY_A, seed=0)
     cfg, w = plain.read_folder(folder, torch.float64)
