@@ -26,6 +26,7 @@ class ModelRunner:
         self.ops = model.ops
         self.vocab_size = model.plan.vocab_size
         self._graphs = None              # width -> captured decode step, once enable_graphs ran
+        self._staging_read = {}          # per captured step: event behind the last copy out of its staging buffer
         self._graph_max = 0
 
     @classmethod
@@ -134,6 +135,9 @@ class ModelRunner:
         if key not in self._graphs:
             self._graphs[key] = self._capture(width, context)
         graph, inputs, staging, logits, _ctx = self._graphs[key]
+        copied = self._staging_read.get(key)
+        if copied is not None:
+            copied.synchronize()            # the last step's copy has read the staging buffer
         host = staging.numpy()
         host[0, n:], host[1, n:], host[2, n:] = 0, 0, cache.null_row
         for i, e in enumerate(entries):
@@ -147,6 +151,9 @@ class ModelRunner:
             host[0, i], host[1, i], host[2, i] = token, start, e.row
         cache.sync()
         inputs.copy_(staging, non_blocking=True)
+        copied = copied or torch.cuda.Event()
+        copied.record()
+        self._staging_read[key] = copied
         graph.replay()
         for e in entries:
             cache.advance(e.row, 1)
