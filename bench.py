@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine at Qwen3-4B size on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--preset qwen3-8b]
 
 A step is one decode step of the engine: plan, run the batch through the model from
 the cache, sample, read the tokens back. Random weights (seeded), prompts of uniform
@@ -22,10 +22,14 @@ sys.path.insert(0, str(ROOT))
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-QWEN3_4B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=2560,
-                num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                intermediate_size=9728, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True)
-FULL_LAYERS = QWEN3_4B["num_hidden_layers"]
+DEFAULT_PRESET = "qwen3-4b"        # socrates_amd/config/presets/qwen3-4b.json: BASELINE.json configs[2]
+
+
+def preset_dict(name):
+    import json
+
+    from socrates_amd.config import preset_path
+    return json.loads(preset_path(name).read_text())
 
 
 def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_):
@@ -58,7 +62,9 @@ def decode_rate(engine, batch, context, steps, warmup, vocab, seed):
     import torch
     rng = random.Random(seed)
     from socrates_amd.sampling import SamplingParams
-    params = SamplingParams(max_new_tokens=batch + warmup + steps + 8, eos_token_ids=())
+    # requests whose prompt is done decode beside the portions of the others: room for that
+    portions = -(-context // engine.scheduler.token_budget)
+    params = SamplingParams(max_new_tokens=batch * portions + warmup + steps + 8, eos_token_ids=())
     reqs = [engine.submit([rng.randrange(vocab) for _ in range(context - 1)], sampling=params)
             for _ in range(batch)]
     while any(not r.output for r in reqs):          # prefill, a portion per step
@@ -106,7 +112,8 @@ def main(argv=None):
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--max-len", type=int, default=4096)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has")
+    ap.add_argument("--preset", default=DEFAULT_PRESET, help="a configuration of socrates_amd/config/presets")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
@@ -121,7 +128,12 @@ def main(argv=None):
     import torch
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     item = 2 if args.dtype == "bf16" else 4
-    cfg = dict(QWEN3_4B, num_hidden_layers=args.layers)
+    cfg = preset_dict(args.preset)
+    full_layers = cfg["num_hidden_layers"]
+    args.layers = args.layers or full_layers
+    cfg["num_hidden_layers"] = args.layers
+    sized = {"qwen3-4b": "Qwen3-4B-sized", "qwen3-8b": "Qwen3-8B-sized", "qwen3-32b": "Qwen3-32B-sized"}.get(
+        args.preset, args.preset)
     biggest = max(args.batch, 1 if args.no_points else 64)
     config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
     V = config.vocab_size
@@ -143,13 +155,13 @@ def main(argv=None):
             points[f"decode_b{b}"] = round(decode_rate(engine, b, args.context, max(8, args.steps // 2),
                                                        4, V, seed=3 + b)[0], 1)
     out = {
-        "metric": "decode tok/s @ batch 8, context 2048 (Qwen3-4B-sized, bf16)",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({sized}, {args.dtype})",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: seeded random weights, uniform random token ids",
-        "config": {"model": "Qwen3-4B-sized", "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single GPU", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": sized, "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_full": full_layers,
                    "hidden_size": config.hidden_size, "num_attention_heads": config.num_attention_heads,
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "intermediate_size": config.intermediate_size, "vocab_size": V,

@@ -44,4 +44,27 @@ def load_config(folder):
     return config_class_for(archs[0]).from_dict(raw)
 
 
+_PRESETS = Path(__file__).resolve().parent / "presets"
+
+
+def known_presets():
+    """Names of the configuration files that come with the package (``presets/*.json``):
+    the two tiny test shapes and Qwen3-4B, -8B and -32B sizes."""
+    return sorted(p.stem for p in _PRESETS.glob("*.json"))
+
+
+def preset_path(name: str) -> Path:
+    path = _PRESETS / f"{name}.json"
+    if not path.is_file():
+        raise ConfigError(f"unknown preset {name!r}; known: {known_presets()}")
+    return path
+
+
+def load_preset(name: str):
+    """The typed configuration of a preset; which class reads it is decided by its own
+    ``architectures`` entry, as for a model folder."""
+    raw = json.loads(preset_path(name).read_text())
+    return config_class_for(raw["architectures"][0]).from_dict(raw)
+
+
 register_architecture("Qwen3ForCausalLM", Qwen3Config)

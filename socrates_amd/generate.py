@@ -36,6 +36,8 @@ def parse_args(argv=None):
                     help="model folder: config.json + model.safetensors (env MODEL_ID)")
     ap.add_argument("--random-weights", metavar="CONFIG_JSON",
                     help="write a random model for this config.json into --model first (seeded by --seed)")
+    ap.add_argument("--preset", help="like --random-weights with a configuration that comes with the package: "
+                                     "tiny-a, tiny-b, qwen3-4b, qwen3-8b, qwen3-32b")
     ap.add_argument("--device", default=os.getenv("DEVICE", "cuda:0"))
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--compile", type=int, default=int(os.getenv("COMPILE", "1") not in ("0", "false", "False")),
@@ -63,6 +65,12 @@ def parse_args(argv=None):
 def main(argv=None) -> int:
     args = parse_args(argv)
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
+    if args.random_weights and args.preset:
+        print("--random-weights and --preset both name a configuration; give one", file=sys.stderr)
+        return 2
+    if args.preset:
+        from .config import preset_path
+        args.random_weights = str(preset_path(args.preset))
     if args.random_weights:
         from .config import config_class_for
         from .weights import write_random_model

@@ -83,6 +83,28 @@ def test_registry(tmp_path):
     assert type(load_config(tmp_path)) is Other
 
 
+def test_presets_that_come_with_the_package():
+    """Five configuration files: the two tiny test shapes and Qwen3-4B, -8B and -32B sizes.
+    Parameter counts of the big ones are the published model sizes; the 4B file says what the
+    reference's pinned copy says, where that is present."""
+    from socrates_amd.config import known_presets, load_preset, preset_path
+    assert known_presets() == ["qwen3-32b", "qwen3-4b", "qwen3-8b", "tiny-a", "tiny-b"]
+    for name, billions in (("qwen3-4b", 4.02), ("qwen3-8b", 8.19), ("qwen3-32b", 32.76)):
+        assert abs(load_preset(name).param_counts()["total"] / 1e9 - billions) < 0.01, name
+    a, b = load_preset("tiny-a"), load_preset("tiny-b")
+    assert (a.head_dim, a.tie_word_embeddings, b.head_dim, b.tie_word_embeddings) == (16, True, 32, False)
+    with pytest.raises(ConfigError, match="unknown preset.*qwen3-4b"):
+        preset_path("qwen3-400b")
+    try:
+        pinned = json.loads(open(REFERENCE_4B).read())
+    except OSError:
+        return
+    ours, theirs = load_preset("qwen3-4b"), Qwen3Config.from_dict(pinned)
+    for key in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads",
+                "head_dim", "intermediate_size", "rms_norm_eps", "rope_theta", "tie_word_embeddings"):
+        assert getattr(ours, key) == getattr(theirs, key), key
+
+
 def test_run_order_is_data():
     plan = Qwen3Config.from_dict(TINY_B["cfg"]).plan()
     fields = {f: getattr(plan, f) for f in plan.__dataclass_fields__}
