@@ -113,3 +113,20 @@ def test_command_line(tmp_path):
     shown = [l for i, l in enumerate(lines) if i > 0 and lines[i - 1].startswith("> ")]
     assert shown == [" ".join(map(str, x)) for x in want]
     assert lines[-1].endswith("tok/s") and "| 10 tok |" in lines[-1]
+
+
+def test_command_line_with_a_preset(tmp_path):
+    """``--preset tiny-b``: the command line writes a seeded random model of that configuration
+    into --model and generates from it; the plain implementation reads the same folder."""
+    folder = tmp_path / "B"
+    cmd = [sys.executable, "-m", "socrates_amd.generate", "--model", str(folder), "--preset", "tiny-b", "--seed", "4",
+           "--dtype", "float32", "--max-new-tokens", "4", "--max-len", "64", "--max-batch", "2", "--block-size", "8",
+           "--prompt-ids", "7,300,12,5,9"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(ROOT))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    cfg, w = plain.read_folder(folder, torch.float64)
+    assert (cfg["num_hidden_layers"], cfg["head_dim"], cfg["vocab_size"]) == (3, 32, 384)
+    want = plain.greedy(cfg, w, [7, 300, 12, 5, 9], 4)
+    lines = proc.stdout.strip().split("\n")
+    shown = [l for i, l in enumerate(lines) if i > 0 and lines[i - 1].startswith("> ")]
+    assert shown == [" ".join(map(str, want))]
