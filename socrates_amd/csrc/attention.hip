@@ -568,7 +568,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 *reinterpret_cast<uint2*>(out + base + j * 16 + 4 * kb) = pk;
             }
         } else {
-            const size_t pi = (base / D) * n_splits + split;
+            // partials lie by (row block, token in it), not by token: a call may cover some of
+            // the tokens only
+            const long shift = row_blocks ? (long)blk * ((16 * RT) >> group_pad_log2) - tok0 : 0;
+            const size_t pi = (size_t)((long)(base / D) + shift * Hq) * n_splits + split;
             if (m[rt] != -INFINITY) {                        // the merge reads nothing of an empty split
 #pragma unroll
                 for (int j = 0; j < DV; ++j)
@@ -586,13 +589,20 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 // group that adds every (64 / (D / 4))-th split, in order; the groups are added in order.
 __global__ void __launch_bounds__(64)
 paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                        bf16* __restrict__ out, int Hq, int n_splits) {
+                        bf16* __restrict__ out, int Hq, int n_splits,
+                        const int* __restrict__ row_blocks, int tokens_per_block) {
     constexpr int LPG = D / 4;                              // lanes of a group
     constexpr int NG = SOC_WAVE / LPG;                      // groups of a wave
     __shared__ float weight[256];
     __shared__ __attribute__((aligned(16))) float4 red[SOC_WAVE];
-    const int h = blockIdx.x, n = blockIdx.y, lane = threadIdx.x;
-    const size_t base = ((size_t)n * Hq + h) * n_splits;
+    const int h = blockIdx.x, lane = threadIdx.x;
+    int n = blockIdx.y;                                     // the token; its partials lie at blockIdx.y
+    if (row_blocks) {
+        const int blk = blockIdx.y / tokens_per_block, j = blockIdx.y % tokens_per_block;
+        if (j >= row_blocks[2 * blk + 1]) return;
+        n = row_blocks[2 * blk] + j;
+    }
+    const size_t base = ((size_t)blockIdx.y * Hq + h) * n_splits;
     constexpr int FAST = 32;                                // partials a lane holds on the short path
     if (n_splits <= SOC_WAVE && n_splits <= FAST * NG) {
         // Few splits: every load is issued before any is needed (one trip to memory instead
@@ -684,8 +694,10 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
 // (16 * row_tiles) >> group_pad_log2 tokens of one sequence, or null: every token is a block
 // of its own (n_row_blocks = N); 2^group_pad_log2 >= min(G, 16).
 // Splits are over absolute key indices: split s covers keys [s * split_len, (s + 1) * split_len),
-// split_len a multiple of 16; n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml
-// [N, Hq, n_splits, 2], which are written for every (row, split), empty ones with m = -inf.
+// split_len a multiple of 16; n_splits > 1 needs part_o [R, Hq, n_splits, D] and part_ml
+// [R, Hq, n_splits, 2] with R = N without row blocks, else n_row_blocks * tokens per block
+// (the blocks may cover some of the N tokens only; the others' outputs are not touched);
+// part_ml is written for every (row, split), empty ones with m = -inf.
 SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const void* v_pool,
                                         const int* block_table, int table_width, const int* token_rows,
                                         const int* positions, const int* row_blocks, int n_row_blocks,
@@ -731,8 +743,11 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
 #undef SOC_MFMA_ARGS
     int err = soc_last_error();
     if (err || n_splits == 1) return err;
-    hipLaunchKernelGGL(paged_attn_merge_kernel, dim3(Hq, N), dim3(64), 0, stream, part_o, part_ml,
-                       (bf16*)out, Hq, n_splits);
+    const int tokens_per_block = (16 * row_tiles) >> group_pad_log2;
+    const long merge_rows = row_blocks ? (long)n_row_blocks * tokens_per_block : (long)N;
+    if (merge_rows > 65535) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(paged_attn_merge_kernel, dim3(Hq, (unsigned)merge_rows), dim3(64), 0, stream, part_o, part_ml,
+                       (bf16*)out, Hq, n_splits, row_blocks, tokens_per_block > 0 ? tokens_per_block : 1);
     return soc_last_error();
 }
 

@@ -358,26 +358,44 @@ class HipKernels:
         split_len = ((max_keys + n - 1) // n + 63) // 64 * 64
         return split_len, (max_keys + split_len - 1) // split_len
 
-    def _row_blocks(self, ctx, n_tokens, tokens_per_block):
-        """int32 [blocks, 2] on the device: (first token, tokens) of each run of at most
-        ``tokens_per_block`` tokens of one sequence; None when every token is a run."""
+    SHORT_PORTION = 16      # sequences of a step with fewer tokens go with the decoded tokens
+
+    @staticmethod
+    def _portion_lengths(ctx):
+        """Tokens of each sequence of the step, or None if the step does not say."""
         import numpy as np
         host = getattr(ctx, "host", None)
-        if host is None or "seq_qstart" not in host or tokens_per_block == 1 or ctx.max_q_len == 1:
+        if host is None or "seq_qstart" not in host:
+            return None
+        qstart = host["seq_qstart"].astype(np.int64)
+        return qstart[1:] - qstart[:-1]
+
+    def _row_blocks(self, ctx, n_tokens, tokens_per_block, which=None):
+        """int32 [blocks, 2] on the device: (first token, tokens) of each run of at most
+        ``tokens_per_block`` tokens of one sequence; None when every token is a run.
+        ``which``: "short" or "long" takes the sequences with fewer than SHORT_PORTION
+        tokens, or the others, only."""
+        import numpy as np
+        lens = self._portion_lengths(ctx)
+        if which is None and (lens is None or tokens_per_block == 1 or ctx.max_q_len == 1):
             # every token alone (always right; what a decode step is anyway): no list
             return None, n_tokens
+        host = ctx.host
         cache = host.setdefault("row_blocks", {})
-        if tokens_per_block not in cache:
-            qstart = host["seq_qstart"].astype(np.int64)
-            lens = qstart[1:] - qstart[:-1]
+        key = (tokens_per_block, which)
+        if key not in cache:
+            qstart = host["seq_qstart"].astype(np.int64)[:-1]
+            if which is not None:
+                keep = (lens < self.SHORT_PORTION) if which == "short" else (lens >= self.SHORT_PORTION)
+                qstart, lens = qstart[keep], lens[keep]
             counts = (lens + tokens_per_block - 1) // tokens_per_block
             seq = np.repeat(np.arange(len(lens)), counts)
             j = np.arange(int(counts.sum())) - np.repeat(np.cumsum(counts) - counts, counts)
             first = qstart[seq] + j * tokens_per_block
             n = np.minimum(tokens_per_block, lens[seq] - j * tokens_per_block)
             blocks = np.stack([first, n], 1).astype(np.int32)
-            cache[tokens_per_block] = (torch.from_numpy(blocks).to(self.device), len(blocks))
-        return cache[tokens_per_block]
+            cache[key] = (torch.from_numpy(blocks).to(self.device), len(blocks))
+        return cache[key]
 
     def plan_mfma(self, n_blocks, n_kv_heads, group, max_keys):
         """(split_len, n_splits) for the MFMA kernel: enough waves to fill the GPU, no split
@@ -391,6 +409,27 @@ class HipKernels:
         n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64))
         split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
         return split_len, (max_keys + split_len - 1) // split_len
+
+    def _wave_attention(self, lib, q, slot, ctx, out, scale, w, rt, gpl, which):
+        """The per-wave MFMA kernel with key splits and merge, for all sequences of the step
+        or for its short ones (``which``), on the current stream."""
+        N, Hq, D = q.shape
+        Hkv = slot.k.shape[1]
+        G = Hq // Hkv
+        tokens_per_block = max(1, (16 * rt) >> gpl)
+        blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block, which)
+        split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_rows = N if blocks is None else n_blocks * tokens_per_block
+            part_o = torch.empty((part_rows, Hq, n_splits, D), dtype=torch.float32, device=self.device)
+            part_ml = torch.empty((part_rows, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
+        _check(lib.soc_paged_attention_mfma(
+            _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+            c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
+            c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), c_int(N), c_int(Hq), c_int(Hkv),
+            c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
+            c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
 
     def paged_attention(self, q, slot, ctx, scale, window=None):
         """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""
@@ -437,35 +476,38 @@ class HipKernels:
             # shorter portion behind a long context is better served by the per-wave kernel
             # with key splits (128 tokens behind 8 k: 95 us against 196 us). An override of
             # the row tiles (tests) forces the choice.
-            enough = (N // wg_tokens) * Hkv * ((G + 15) // 16) >= 256 or self.attention_row_tiles is not None
+            # A step that mixes long portions with decoded tokens (or short ends of prompts):
+            # the long ones to the workgroup kernel, the short ones to the per-wave kernel,
+            # whose key splits a single token behind a long context needs (in the workgroup
+            # kernel it would hold four waves and walk its whole context alone).
+            lens = self._portion_lengths(ctx)
+            mixed = (not decode and lens is not None and bool((lens < self.SHORT_PORTION).any())
+                     and bool((lens >= self.SHORT_PORTION).any()))
+            n_long = int(lens[lens >= self.SHORT_PORTION].sum()) if mixed else N
+            enough = (n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= 256 or self.attention_row_tiles is not None
+            which = None
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt
                 self.last_attention_kernel = ("workgroup", rt)
-                blocks, n_blocks = self._row_blocks(ctx, N, wg_tokens)
+                blocks, n_blocks = self._row_blocks(ctx, N, wg_tokens, "long" if mixed else None)
                 _check(lib.soc_paged_attention_prefill(
                     _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
                     c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
                     c_int(n_blocks), _ptr(out), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
                     c_float(scale), c_int(w), c_int(rt), c_int(gpl), self._stream()),
                     "paged_attention (prefill)")
+                if not mixed:
+                    return out
+                which = "short"
+                # after the long ones, on the same stream: side by side on a second stream was
+                # measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)
+                self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, which)
                 return out
             rt = self.attention_row_tiles or 1
             rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
-            tokens_per_block = max(1, (16 * rt) >> gpl)
             self.last_attention_kernel = ("wave", rt)
-            blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block)
-            split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
-            part_o = part_ml = None
-            if n_splits > 1:
-                part_o = torch.empty((N, Hq, n_splits, D), dtype=torch.float32, device=self.device)
-                part_ml = torch.empty((N, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
-            _check(lib.soc_paged_attention_mfma(
-                _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
-                c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
-                c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), c_int(N), c_int(Hq), c_int(Hkv),
-                c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
-                c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
+            self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None)
             return out
         max_keys = ctx.max_ctx_len if not w else min(w, ctx.max_ctx_len)
         split_len, n_splits = self.plan_splits(N, Hkv, G, max_keys)
