@@ -396,27 +396,29 @@ def test_qk_norm_rope_write(kernel_sets, dtype, Hq, Hkv, D, rot):
     close(fresh.slot(0).k, caches[1].slot(0).k, dtype)
 
 
+@pytest.mark.parametrize("n0", [200, 900])
 @pytest.mark.parametrize("Hq,Hkv,D,rope", [(32, 8, 128, True), (5, 1, 128, True), (6, 2, 64, True), (9, 3, 64, False),
                                            (4, 2, 128, False)])
-def test_qk_norm_rope_write_long_prompts(kernel_sets, Hq, Hkv, D, rope):
+def test_qk_norm_rope_write_long_prompts(kernel_sets, Hq, Hkv, D, rope, n0):
     """Hundreds of tokens in bfloat16 take the kernel that works on several heads per wave
-    (head sizes 64 and 128, rotation over the whole head or none); head counts that do not
-    fill the last wave, two rows, one of them continuing at position 37."""
+    (head sizes 64 and 128, rotation over the whole head or none), from 1,024 tokens on its
+    form with a token per wave (1,031 tokens: the last workgroup has three); head counts that
+    do not fill the last wave, two rows, one of them continuing at position 37."""
     from socrates_amd.cache import CacheManager
     from socrates_amd.parts import PagedKV
     dtype = torch.bfloat16
     hip, ref = kernel_sets[dtype]
     bs = 16
-    caches = [CacheManager([PagedKV(Hkv, D)], 2, 512, bs, 40, dtype, DEV) for _ in range(2)]
+    caches = [CacheManager([PagedKV(Hkv, D)], 2, 1024, bs, 80, dtype, DEV) for _ in range(2)]
     for c in caches:
         r0, r1 = c.open_row(), c.open_row()
-        c.reserve(r0, 200)
+        c.reserve(r0, n0)
         c.reserve(r1, 37)
         c.advance(r1, 37)
         c.reserve(r1, 37 + 131)
         c.sync()
-    rows = [0] * 200 + [1] * 131
-    pos = list(range(200)) + list(range(37, 37 + 131))
+    rows = [0] * n0 + [1] * 131
+    pos = list(range(n0)) + list(range(37, 37 + 131))
     N = len(rows)
     positions = torch.tensor(pos, dtype=torch.int32, device=DEV)
     token_rows = torch.tensor(rows, dtype=torch.int32, device=DEV)
