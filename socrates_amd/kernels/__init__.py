@@ -450,22 +450,38 @@ class HipKernels:
             decode = getattr(ctx, "max_q_len", 1) == 1
             if N > 65535:
                 raise KernelError("more than 65535 tokens in one attention call")
-            # row tiles 32: 32 rows per wave through the 32 x 32 products (head sizes in steps of 32)
-            # 64: the same with eight waves, each four on one half of a block's keys
+            # A step that mixes long portions with decoded tokens (or short ends of prompts):
+            # the long ones go to the workgroup kernel, the short ones to the per-wave kernel,
+            # whose key splits a single token behind a long context needs (in the workgroup
+            # kernel it would hold four waves and walk its whole context alone).
+            lens = self._portion_lengths(ctx)
+            long_ = None if lens is None else lens >= self.SHORT_PORTION
+            mixed = not decode and long_ is not None and bool(long_.any()) and not bool(long_.all())
+            n_long = int(lens[long_].sum()) if mixed else N
+            # even: no row of a long portion sees less than half the keys that another sees
+            seq_ctx = None if lens is None else ctx.host.get("seq_ctx")
+            if seq_ctx is not None and long_.any():
+                even = bool((seq_ctx[long_] >= 2 * lens[long_]).all())
+            else:
+                even = ctx.max_ctx_len >= 2 * getattr(ctx, "max_q_len", 1)
+            # Row tiles of the workgroup kernel. 1, 2: 16 or 32 rows per wave through the
+            # 16 x 16 products; 32: 32 rows per wave through the 32 x 32 products (head sizes
+            # in steps of 32); 64: the same with eight waves, each four on one half of a
+            # block's keys.
             wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2, 32, 64) else (2 if D <= 64 else 1)
             if wg_rt >= 32 and D % 32:
                 wg_rt = 1
             if self.attention_row_tiles is None and D > 64 and D % 32 == 0:
                 # head sizes 96 and 128 (64 and less hold two row tiles anyway): 20 % faster
                 # where its workgroups, half as many, still fill the GPU evenly: two for every
-                # slot (512 of four waves), or one if no row sees less than half the keys of
-                # another. Uneven and one per slot (a prompt of 2,048 tokens from its start):
-                # the eight-wave form, which splits each block's keys inside the workgroup.
+                # slot (512 of four waves), or one if the work is even. Uneven and one per slot
+                # (a prompt of 2,048 tokens from its start): the eight-wave form, which splits
+                # each block's keys inside the workgroup.
                 # Measured at 8 kv heads of 4 x 128, 16 / 32 / 32 rows in two halves:
                 # 2,048 tokens behind 6,144: 436 / 355 / 376 us; 4,096 from 0: 267 / 222 / 241;
                 # 2,048 from 0: 91 / 88 / 78; 1,024 from 0: 34 / 43 / 36.
-                n32 = (N // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16)
-                if n32 >= 1024 or (n32 >= 512 and ctx.max_ctx_len >= 2 * getattr(ctx, "max_q_len", 1)):
+                n32 = (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16)
+                if n32 >= 1024 or (n32 >= 512 and even):
                     wg_rt = 32
                 elif n32 >= 512:
                     wg_rt = 64
@@ -476,16 +492,7 @@ class HipKernels:
             # shorter portion behind a long context is better served by the per-wave kernel
             # with key splits (128 tokens behind 8 k: 95 us against 196 us). An override of
             # the row tiles (tests) forces the choice.
-            # A step that mixes long portions with decoded tokens (or short ends of prompts):
-            # the long ones to the workgroup kernel, the short ones to the per-wave kernel,
-            # whose key splits a single token behind a long context needs (in the workgroup
-            # kernel it would hold four waves and walk its whole context alone).
-            lens = self._portion_lengths(ctx)
-            mixed = (not decode and lens is not None and bool((lens < self.SHORT_PORTION).any())
-                     and bool((lens >= self.SHORT_PORTION).any()))
-            n_long = int(lens[lens >= self.SHORT_PORTION].sum()) if mixed else N
             enough = (n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= 256 or self.attention_row_tiles is not None
-            which = None
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt
@@ -497,12 +504,10 @@ class HipKernels:
                     c_int(n_blocks), _ptr(out), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
                     c_float(scale), c_int(w), c_int(rt), c_int(gpl), self._stream()),
                     "paged_attention (prefill)")
-                if not mixed:
-                    return out
-                which = "short"
-                # after the long ones, on the same stream: side by side on a second stream was
-                # measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)
-                self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, which)
+                if mixed:
+                    # after the long ones, on the same stream: side by side on a second stream
+                    # was measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)
+                    self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, "short")
                 return out
             rt = self.attention_row_tiles or 1
             rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
