@@ -307,6 +307,8 @@ __device__ __forceinline__ uint4 load_qk_slice(const bf16* row, int kk, int kb) 
 }
 
 // TP: pages hold a multiple of 16 keys (and a power of two of them), so a tile lies in one page.
+constexpr float LAZY_MAX = 8.f;        // log2 of the largest softmax weight before a row's reference moves
+
 template <int RT, bool TP>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
@@ -454,10 +456,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             for (int kk = 0; kk < QK_STEPS; ++kk)
                 s = qk_mfma(k_ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u), qf[rt][kk], s);
             float sv[4];
-            float mx = -INFINITY;
+            float mx = -INFINITY;                           // of the raw scores: the scale is positive
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                sv[r] = s[r] * c2;
+                sv[r] = s[r];
                 if constexpr (MASKED) {
                     const int key = key0 + 4 * kb + r;
                     bool seen = key <= row_pos[rt] && key < khi && key >= split * split_len;
@@ -466,19 +468,24 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 }
                 mx = fmaxf(mx, sv[r]);
             }
-            mx = max_xor32(max_xor16(mx));
-            const float mn = fmaxf(m[rt], mx);
-            const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
-            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - ms);
+            mx = max_xor32(max_xor16(mx)) * c2;
+            // m is the row's reference for the exponentials, not its maximum: it moves only
+            // when a tile's maximum lies more than LAZY_MAX above it, so the accumulators are
+            // rescaled a few times per row instead of in most tiles (weights stay below 2^8);
+            // the merge of splits works with any reference
+            const bool move = mx > m[rt] + LAZY_MAX;
+            const float mn = move ? mx : m[rt];
+            const float ms = mn == -INFINITY ? 0.f : mn;
+            alpha[rt] = move ? __builtin_amdgcn_exp2f(m[rt] - ms) : 1.f;
             float p[4];
             float psum = 0.f;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(sv[r] - ms);
+                p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[r], c2, -ms));
                 psum += p[r];
             }
             l[rt] = l[rt] * alpha[rt] + psum;
-            any_rescale = any_rescale || (m[rt] != mn);
+            any_rescale = any_rescale || move;
             m[rt] = mn;
             const uint32_t p01 = pack_bf16x2(p[0], p[1]), p23 = pack_bf16x2(p[2], p[3]);
             pf[rt] = (s16x4_t){(short)(p01 & 0xffffu), (short)(p01 >> 16), (short)(p23 & 0xffffu), (short)(p23 >> 16)};
@@ -712,6 +719,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
     if (n_splits > 256) return (int)hipErrorInvalidValue;        // the merge holds 256 weights
+    if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     const dim3 grid((unsigned)((tasks + 3) / 4), n_splits);
     int bs_shift = -1;                                           // log2 of the page size if it is a power of two
@@ -979,10 +987,10 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                 s1 = qk_mfma(kc[kk], qf[rt][kk], s1);
             }
             float t[8];
-            float mx = -INFINITY;
+            float mx = -INFINITY;                           // of the raw scores: the scale is positive
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                t[r] = (r < 4 ? s0[r & 3] : s1[r & 3]) * c2;
+                t[r] = r < 4 ? s0[r & 3] : s1[r & 3];
                 if constexpr (MASKED) {
                     const int key = key0 + 8 * kb + r;
                     bool seen = key <= row_pos[rt];
@@ -991,19 +999,22 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                 }
                 mx = fmaxf(mx, t[r]);
             }
-            mx = max_xor32(max_xor16(mx));
-            const float mn = fmaxf(m[rt], mx);
-            const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
-            alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - ms);
+            mx = max_xor32(max_xor16(mx)) * c2;
+            // m is the row's reference for the exponentials, moved only when a tile's maximum
+            // lies more than LAZY_MAX above it (see the 32-row form)
+            const bool move = mx > m[rt] + LAZY_MAX;
+            const float mn = move ? mx : m[rt];
+            const float ms = mn == -INFINITY ? 0.f : mn;
+            alpha[rt] = move ? __builtin_amdgcn_exp2f(m[rt] - ms) : 1.f;
             float p[8];
             float psum = 0.f;
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(t[r] - ms);
+                p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(t[r], c2, -ms));
                 psum += p[r];
             }
             l[rt] = l[rt] * alpha[rt] + psum;
-            any_rescale = any_rescale || (m[rt] != mn);
+            any_rescale = any_rescale || move;
             m[rt] = mn;
             pf[rt] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
                                 pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
@@ -1050,32 +1061,33 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t*>(&ka),
                                                          *reinterpret_cast<const bf16x8_t*>(&qa), sc, 0, 0, 0);
         }
-        float tv[16];
-        float mx = -INFINITY;
+        float mx = -INFINITY;                               // of the raw scores: the scale is positive
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            tv[i] = sc[i] * c2;
             if constexpr (MASKED) {
                 const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
                 bool seen = key <= row_pos32;
                 if (window > 0) seen = seen && key > row_pos32 - window;
-                tv[i] = seen ? tv[i] : -INFINITY;
+                sc[i] = seen ? sc[i] : -INFINITY;
             }
-            mx = fmaxf(mx, tv[i]);
+            mx = fmaxf(mx, sc[i]);
         }
-        mx = max_xor32(mx);
-        const float mn = fmaxf(m32, mx);
-        const float ms = (MASKED && mn == -INFINITY) ? 0.f : mn;
-        const float alpha = __builtin_amdgcn_exp2f(m32 - ms);
+        mx = max_xor32(mx) * c2;
+        // m32 is the row's reference for the exponentials, not its maximum: it moves only when
+        // a tile's maximum lies more than LAZY_MAX above it, so the accumulators are rescaled a
+        // few times per row instead of in most tiles; weights stay below 2^LAZY_MAX
+        const bool rescale = mx > m32 + LAZY_MAX;
+        const float mn = rescale ? mx : m32;
+        const float ms = mn == -INFINITY ? 0.f : mn;
+        const float alpha = rescale ? __builtin_amdgcn_exp2f(m32 - ms) : 1.f;
         float p[16];
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            p[i] = __builtin_amdgcn_exp2f(tv[i] - ms);
+            p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c2, -ms));
             psum += p[i];
         }
         l32 = l32 * alpha + psum;
-        const bool rescale = m32 != mn;
         m32 = mn;
         uint4 pf[2];
 #pragma unroll
@@ -1230,6 +1242,7 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
                                            hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1) return (int)hipErrorInvalidValue;
+    if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;

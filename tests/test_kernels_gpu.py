@@ -296,6 +296,40 @@ def test_prefill_attention_long_portions_choose_the_32_row_products(kernel_sets,
     assert (got[700].view(Hq, D)[37].float().cpu() - v0[37 // 16, 3]).abs().max() < 0.05
 
 
+@pytest.mark.parametrize("rise", [0.004, 0.05, -0.05])
+def test_attention_scores_that_keep_rising(kernel_sets, rise):
+    """Keys whose scores rise (or fall) steadily along the sequence: the running reference of
+    the softmax has to follow, by small steps that stay under the threshold up to which the
+    MFMA kernels leave it where it is (0.004: 7 bits over 600 keys; 0.05: 86 bits, a move every
+    few tiles; -0.05: it stays at the first tile's), for a decoded token with and without key splits and for a prompt portion
+    through every form of the workgroup kernel."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    Hq, Hkv, D, bs, n = 8, 2, 64, 16, 600
+    slot, dense = make_paged_case([n], Hq, Hkv, D, bs, torch.bfloat16, seed=3)
+    g = torch.Generator().manual_seed(8)
+    direction = torch.nn.functional.normalize(torch.randn(Hkv, D, generator=g), dim=-1)
+    # key j of head h = noise + 8 rise j direction[h]; q = 2 direction[h] + noise: score 2 rise j, times log2 e in bits
+    k_new = (0.1 * torch.randn(Hkv, n, D, generator=g) + rise * torch.arange(n)[None, :, None] * direction[:, None] * 8).to(torch.bfloat16)
+    table = slot.block_table[0].tolist()
+    for j in range(n):
+        slot.k[table[j // bs], :, j % bs] = k_new[:, j].to(DEV)
+    dense[0] = (k_new.float(), dense[0][1])
+    q = (direction.repeat_interleave(Hq // Hkv, 0)[None] * 2 + 0.05 * torch.randn(40, Hq, D, generator=g)).to(torch.bfloat16).to(DEV)
+    # a decoded token at the end
+    want = dense_attention(q[:1], dense, [0], [n - 1], D ** -0.5)
+    for splits in (None, (64, 10), (1 << 30, 1)):
+        hip.attention_splits = splits
+        close(hip.paged_attention(q[:1].contiguous(), slot, ctx_for([0], [n - 1]), D ** -0.5).cpu(), want, torch.bfloat16)
+    hip.attention_splits = None
+    # a portion of 40 tokens at the end
+    rows, pos = [0] * 40, list(range(n - 40, n))
+    want = dense_attention(q, dense, rows, pos, D ** -0.5)
+    for rt in (1, 2, 32, 64):
+        hip.attention_row_tiles = rt
+        close(hip.paged_attention(q, slot, ctx_for(rows, pos), D ** -0.5).cpu(), want, torch.bfloat16)
+    hip.attention_row_tiles = None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n,slot_idx", [(1, 0), (16, 15), (17, 16), (256, 255), (257, 256), (1024, 1023),
                                         (1, 1), (15, 15), (16, 16), (255, 255), (256, 256), (1024, 1024),
