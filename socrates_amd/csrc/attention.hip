@@ -309,6 +309,27 @@ __device__ __forceinline__ uint4 load_qk_slice(const bf16* row, int kk, int kb) 
 // TP: pages hold a multiple of 16 keys (and a power of two of them), so a tile lies in one page.
 constexpr float LAZY_MAX = 8.f;        // log2 of the largest softmax weight before a row's reference moves
 
+// The rare tile that moves a reference rescales the accumulators where they are, one register
+// at a time, each multiply written so that the compiler cannot regroup it: a product that
+// defines a whole accumulator anew gives it a new home, and then every tile copies all
+// accumulators at the join behind the branch, rescaled or not.
+__device__ __forceinline__ void scale_in_place(float& v, float by) {
+    asm volatile("v_mul_f32 %0, %0, %1" : "+v"(v) : "v"(by));
+}
+template <int RT_, int DV_>
+__device__ __forceinline__ void rescale_in_place(f32x4_t (&o)[RT_][DV_], const float (&alpha)[RT_]) {
+#pragma unroll
+    for (int rt = 0; rt < RT_; ++rt)
+#pragma unroll
+        for (int j = 0; j < DV_; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float v = o[rt][j][e];
+                scale_in_place(v, alpha[rt]);
+                o[rt][j][e] = v;
+            }
+}
+
 template <int RT, bool TP>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
@@ -425,7 +446,12 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 
     // One tile: V to LDS, scores, online softmax, weighted values. MASKED: some key of the
     // tile is hidden from some row of the block (or lies outside the split).
-    auto compute = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE], auto masked_tag) {
+    // A tile in two halves. The first (MASKED or not): the V tile to LDS, scores and softmax
+    // weights, packed as operand B of the second product. The second half is one piece of code
+    // behind both variants, so that the accumulators have one home (with the products inside
+    // the variants the compiler copies accumulators at every join).
+    auto scores = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE], auto masked_tag,
+                      s16x4_t (&pf)[RT], float (&alpha)[RT], bool& any_rescale) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk); keys
         // that were not to be read become zeros here, now that their loads have landed
@@ -446,9 +472,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         }
         __builtin_amdgcn_wave_barrier();
         const bool k_ok = !MASKED || (key0 + li >= kmin && key0 + li < khi);
-        s16x4_t pf[RT];
-        bool any_rescale = false;
-        float alpha[RT];
+        any_rescale = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             f32x4_t s = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -490,12 +514,9 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             const uint32_t p01 = pack_bf16x2(p[0], p[1]), p23 = pack_bf16x2(p[2], p[3]);
             pf[rt] = (s16x4_t){(short)(p01 & 0xffffu), (short)(p01 >> 16), (short)(p23 & 0xffffu), (short)(p23 >> 16)};
         }
-        if (__any(any_rescale)) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
-        }
+    };
+    auto weighted = [&](const s16x4_t (&pf)[RT], const float (&alpha)[RT], bool any_rescale) {
+        if (__any(any_rescale)) rescale_in_place(o, alpha);
         // O^T += V^T P^T, one 16-wide block of d at a time; the V^T slice is shared by the row tiles
 #pragma unroll
         for (int j = 0; j < DV; ++j) {
@@ -514,12 +535,16 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     auto tile = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE]) {
         const bool whole = key0 >= split * split_len && key0 + 15 < khi && key0 + 15 <= pos0 &&
                            (window <= 0 || key0 > last_pos - window);
+        s16x4_t pf[RT];
+        float alpha[RT];
+        bool any_rescale;
         if constexpr (D > 128) {
-            compute(key0, kf, vr, std::true_type{});         // one variant: registers are short at these sizes
+            scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale);     // one variant: registers are short at these sizes
         } else {
-            if (whole) compute(key0, kf, vr, std::false_type{});
-            else compute(key0, kf, vr, std::true_type{});
+            if (whole) scores(key0, kf, vr, std::false_type{}, pf, alpha, any_rescale);
+            else scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale);
         }
+        weighted(pf, alpha, any_rescale);
     };
 
     // Three tiles are in flight per wave (48 keys). Buffer b holds tiles b, b + 3, b + 6, ...
@@ -794,7 +819,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
 // PAIR: pages hold an even, power-of-two number of keys, so a thread's two keys share a page.
 // M32: a wave owns 32 rows and multiplies with the 32 x 32 x 16 instruction (RT = 1; head
-// sizes that are multiples of 32): per row, half the loads, LDS reads, stores and barriers.
+// sizes that are multiples of 32): per row, half the loads, LDS reads, stores and barriers
+// of RT = 1, as RT = 2 has with the 16 x 16 products; the two are equally fast.
 // KS = 2 (with M32): eight waves; waves 0-3 walk the first half of the block's key tiles and
 // waves 4-7, with the same rows, the second half, each four with tiles of their own in LDS;
 // at the end the two partial results are combined through LDS. Twice the waves for the same
@@ -874,11 +900,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int c32 = lane % 32, g32 = lane / 32;
     int row_pos32 = -1;
     size_t row_q32 = 0;
-    // the lane's slices of its query row wait in LDS (each lane reads back what it wrote):
-    // with them in registers a wave would need more than half of a SIMD's registers
-    __shared__ __align__(16) uint16_t q_lds[M32 ? KS * 4 * 32 * PF_K_STRIDE : 8];
-    const int q_off = M32 ? (wave_all * 32 + c32) * PF_K_STRIDE + 8 * g32 : 0;
-    uint16_t* q_mine = q_lds + q_off;
+    uint4 qf32[M32 ? DQ32 : 1];                           // the lane's slices of its query row
     f32x16_t o32[M32 ? DB32 : 1];
     float m32 = -INFINITY, l32 = 0.f;
     if constexpr (M32) {
@@ -888,8 +910,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         row_q32 = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? gh : 0)) * D;
 #pragma unroll
         for (int t = 0; t < DQ32; ++t)
-            *reinterpret_cast<uint4*>(q_mine + 16 * t) =
-                ok ? *reinterpret_cast<const uint4*>(q + row_q32 + 16 * t + 8 * g32) : make_uint4(0u, 0u, 0u, 0u);
+            qf32[t] = ok ? *reinterpret_cast<const uint4*>(q + row_q32 + 16 * t + 8 * g32) : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
         for (int b = 0; b < DB32; ++b)
 #pragma unroll
@@ -964,20 +985,21 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         }
     };
 
-    // One tile for this wave's rows. MASKED: some key of the tile is hidden from some row.
-    auto compute = [&](int key0, int buf, auto masked_tag) {
+    // One tile for this wave's rows, in two halves. The first: scores and softmax weights
+    // (packed as operand B of the second product); MASKED: some key of the tile is hidden from
+    // some row. The second half is one piece of code behind both variants, so that the
+    // accumulators have one home: with the products inside the variants the compiler copied
+    // all accumulators at every join.
+    auto scores = [&](int key0, int buf, auto masked_tag, uint4 (&pf)[RT], float (&alpha)[RT], bool& any_rescale) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         const uint16_t* kt = k_lds[buf];
-        const uint16_t* vt = v_lds[buf];
         uint4 ka[QK_STEPS], kc[QK_STEPS];
 #pragma unroll
         for (int kk = 0; kk < QK_STEPS; ++kk) {
             ka[kk] = load_qk_slice(reinterpret_cast<const bf16*>(kt + li * PF_K_STRIDE), kk, kb);
             kc[kk] = load_qk_slice(reinterpret_cast<const bf16*>(kt + (16 + li) * PF_K_STRIDE), kk, kb);
         }
-        uint4 pf[RT];
-        float alpha[RT];
-        bool any_rescale = false;
+        any_rescale = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             f32x4_t s0 = (f32x4_t){0.f, 0.f, 0.f, 0.f}, s1 = s0;
@@ -1019,12 +1041,10 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             pf[rt] = make_uint4(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]),
                                 pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
         }
-        if (__any(any_rescale)) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                for (int j = 0; j < DV; ++j) o[rt][j] *= alpha[rt];
-        }
+    };
+    auto weighted = [&](int buf, const uint4 (&pf)[RT], const float (&alpha)[RT], bool any_rescale) {
+        const uint16_t* vt = v_lds[buf];
+        if (__any(any_rescale)) rescale_in_place(o, alpha);
         // O^T += V^T P^T over the 32 keys, one 16-wide block of d at a time
         uint4 va[DV];
 #pragma unroll
@@ -1044,22 +1064,17 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 
     // The same with 32 rows per wave: S^T [32 keys x 32 rows] from D / 16 products, a row's
     // scores in two lanes (16 each), O^T [32 d x 32 rows] per 32-wide block of d.
-    auto compute32 = [&](int key0, int buf, auto masked_tag) {
+    auto scores32 = [&](int key0, int buf, auto masked_tag, uint4 (&pf)[2], float& alpha, bool& rescale) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         const uint16_t* kt = k_lds[buf];
-        const uint16_t* vt = v_lds[buf];
         f32x16_t sc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[i] = 0.f;
-        int q_at = q_off;
-        asm volatile("" : "+v"(q_at));                      // read every tile anew: not hoisted back into registers
-        const uint16_t* q_mine = q_lds + q_at;
 #pragma unroll
         for (int t = 0; t < DQ32; ++t) {
             const uint4 ka = *reinterpret_cast<const uint4*>(kt + c32 * PF_K_STRIDE + 16 * t + 8 * g32);
-            const uint4 qa = *reinterpret_cast<const uint4*>(q_mine + 16 * t);
             sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t*>(&ka),
-                                                         *reinterpret_cast<const bf16x8_t*>(&qa), sc, 0, 0, 0);
+                                                         *reinterpret_cast<const bf16x8_t*>(&qf32[t]), sc, 0, 0, 0);
         }
         float mx = -INFINITY;                               // of the raw scores: the scale is positive
 #pragma unroll
@@ -1076,10 +1091,10 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         // m32 is the row's reference for the exponentials, not its maximum: it moves only when
         // a tile's maximum lies more than LAZY_MAX above it, so the accumulators are rescaled a
         // few times per row instead of in most tiles; weights stay below 2^LAZY_MAX
-        const bool rescale = mx > m32 + LAZY_MAX;
+        rescale = mx > m32 + LAZY_MAX;
         const float mn = rescale ? mx : m32;
         const float ms = mn == -INFINITY ? 0.f : mn;
-        const float alpha = rescale ? __builtin_amdgcn_exp2f(m32 - ms) : 1.f;
+        alpha = rescale ? __builtin_amdgcn_exp2f(m32 - ms) : 1.f;
         float p[16];
         float psum = 0.f;
 #pragma unroll
@@ -1089,14 +1104,22 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         }
         l32 = l32 * alpha + psum;
         m32 = mn;
-        uint4 pf[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h)
             pf[h] = make_uint4(pack_bf16x2(p[8 * h], p[8 * h + 1]), pack_bf16x2(p[8 * h + 2], p[8 * h + 3]),
                                pack_bf16x2(p[8 * h + 4], p[8 * h + 5]), pack_bf16x2(p[8 * h + 6], p[8 * h + 7]));
-        if (__any(rescale)) {
+    };
+    auto weighted32 = [&](int buf, const uint4 (&pf)[2], float alpha, bool rescale) {
+        const uint16_t* vt = v_lds[buf];
+        if (__any(rescale)) {                               // rare; in place (see scale_in_place)
 #pragma unroll
-            for (int b = 0; b < DB32; ++b) o32[b] *= alpha;
+            for (int b = 0; b < DB32; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    float v = o32[b][i];
+                    scale_in_place(v, alpha);
+                    o32[b][i] = v;
+                }
         }
 #pragma unroll
         for (int b = 0; b < DB32; ++b) {
@@ -1128,11 +1151,19 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             const bool whole = key0 + PF_KEYS - 1 <= wave_lo_pos &&
                                (window <= 0 || key0 > wave_hi_pos - window);
             if constexpr (M32) {
-                if (whole) compute32(key0, buf, std::false_type{});
-                else compute32(key0, buf, std::true_type{});
+                uint4 pf[2];
+                float alpha;
+                bool rescale;
+                if (whole) scores32(key0, buf, std::false_type{}, pf, alpha, rescale);
+                else scores32(key0, buf, std::true_type{}, pf, alpha, rescale);
+                weighted32(buf, pf, alpha, rescale);
             } else {
-                if (whole) compute(key0, buf, std::false_type{});
-                else compute(key0, buf, std::true_type{});
+                uint4 pf[RT];
+                float alpha[RT];
+                bool any_rescale;
+                if (whole) scores(key0, buf, std::false_type{}, pf, alpha, any_rescale);
+                else scores(key0, buf, std::true_type{}, pf, alpha, any_rescale);
+                weighted(buf, pf, alpha, any_rescale);
             }
         }
     };
