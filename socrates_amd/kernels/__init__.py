@@ -458,33 +458,30 @@ class HipKernels:
             long_ = None if lens is None else lens >= self.SHORT_PORTION
             mixed = not decode and long_ is not None and bool(long_.any()) and not bool(long_.all())
             n_long = int(lens[long_].sum()) if mixed else N
-            # even: no row of a long portion sees less than half the keys that another sees
-            seq_ctx = None if lens is None else ctx.host.get("seq_ctx")
-            if seq_ctx is not None and long_.any():
-                even = bool((seq_ctx[long_] >= 2 * lens[long_]).all())
-            else:
-                even = ctx.max_ctx_len >= 2 * getattr(ctx, "max_q_len", 1)
             # Row tiles of the workgroup kernel. 1, 2: 16 or 32 rows per wave through the
             # 16 x 16 products; 32: 32 rows per wave through the 32 x 32 products (head sizes
             # in steps of 32); 64: the same with eight waves, each four on one half of a
-            # block's keys.
-            wg_rt = self.attention_row_tiles if self.attention_row_tiles in (1, 2, 32, 64) else (2 if D <= 64 else 1)
-            if wg_rt >= 32 and D % 32:
-                wg_rt = 1
-            if self.attention_row_tiles is None and D > 64 and D % 32 == 0:
-                # head sizes 96 and 128 (64 and less hold two row tiles anyway): 20 % faster
-                # where its workgroups, half as many, still fill the GPU evenly: two for every
-                # slot (512 of four waves), or one if the work is even. Uneven and one per slot
-                # (a prompt of 2,048 tokens from its start): the eight-wave form, which splits
-                # each block's keys inside the workgroup.
-                # Measured at 8 kv heads of 4 x 128, 16 / 32 / 32 rows in two halves:
-                # 2,048 tokens behind 6,144: 436 / 355 / 376 us; 4,096 from 0: 267 / 222 / 241;
-                # 2,048 from 0: 91 / 88 / 78; 1,024 from 0: 34 / 43 / 36.
+            # block's keys. Chosen by the number of 32-row workgroups the long portions give
+            # (measured at 8 kv heads of 4 x 128 and 4 x 64, in us for 16 / 2 x 16 / 32 rows /
+            # 32 rows in two key halves; 512 slots of four waves on the GPU):
+            #   256 tokens from 0 (64 workgroups): 11 / 14 / 13 / 14;  512 (128): 17 / 21 / 20 / 19
+            #   1,024 from 0 (256): 32 / 36 / 34 / 29;  2,048 (512): 82 / 74 / 69 / 62
+            #   3,072 from 0 (768): 163 / 112 / 107 / 123;  8,192 (2,048): 941 / 650 / 633 / 695
+            #   1,024 behind 3,072 (256): 117 / 122 / 111 / 89;  2,048 behind 6,144 (512): 488 / 305 / 296 / 297
+            # at head size 64 the eight-wave form stays ahead or level up to 8,192 tokens.
+            wg_rt = 1
+            if self.attention_row_tiles in (1, 2, 32, 64):
+                wg_rt = self.attention_row_tiles
+                if wg_rt >= 32 and D % 32:
+                    wg_rt = 1
+            elif D % 32 == 0:
                 n32 = (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16)
-                if n32 >= 1024 or (n32 >= 512 and even):
+                if n32 >= 768 and D > 64:
                     wg_rt = 32
-                elif n32 >= 512:
+                elif n32 >= 256:
                     wg_rt = 64
+            elif D <= 64 and (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16) >= 512:
+                wg_rt = 2
             wg_tokens = 4 * max(1, (32 if wg_rt >= 32 else 16 * wg_rt) >> gpl)
             # Prompt portions go to the kernel whose four waves share the K and V tiles, if it
             # has a workgroup for every compute unit (it has no key splits; measured: 512

@@ -275,15 +275,14 @@ def test_prefill_attention_whole_prompts(kernel_sets, Hq, Hkv, D, bs):
     hip.attention_row_tiles = None
 
 
-@pytest.mark.parametrize("start,row_tiles", [(1024, 32), (0, 64)])
-def test_prefill_attention_long_portions_choose_the_32_row_products(kernel_sets, start, row_tiles):
-    """Portions long enough that head size 128 goes to the 32-row products by itself (512
-    workgroups of 8 tokens x 16 heads of a group): behind a context, where every row sees at
-    least half the keys that the last one sees, with four waves; from the start of a prompt
-    with eight, each four on half of the keys. One early key is made to stand out for one query."""
+@pytest.mark.parametrize("start,T,row_tiles", [(1024, 1024, 64), (0, 1024, 64), (0, 1536, 32)])
+def test_prefill_attention_long_portions_choose_the_32_row_products(kernel_sets, start, T, row_tiles):
+    """Portions long enough that head size 128 goes to the 32-row products by itself
+    (workgroups of 8 tokens x 16 heads of a group): 512 of them take the eight-wave form,
+    each four waves on half of the keys, behind a context or from the start of a prompt; 768
+    the four-wave form. One early key is made to stand out for one query."""
     hip, _ = kernel_sets[torch.bfloat16]
     Hq, Hkv, D, bs = 64, 4, 128, 16
-    T = 1024
     slot, dense = make_paged_case([start + T], Hq, Hkv, D, bs, torch.bfloat16, seed=5)
     rows, pos = [0] * T, list(range(start, start + T))
     q = rnd((T, Hq, D), torch.bfloat16, 22)
