@@ -316,8 +316,13 @@ constexpr float LAZY_MAX = 8.f;        // log2 of the largest softmax weight bef
 __device__ __forceinline__ void scale_in_place(float& v, float by) {
     asm volatile("v_mul_f32 %0, %0, %1" : "+v"(v) : "v"(by));
 }
+// The compiler does not look into these multiplies when it places the wait states that a
+// matrix instruction needs after (or before) a vector instruction on the same registers; a
+// rescaling is rare, so it is simply fenced with more idle cycles than any such rule asks for.
+__device__ __forceinline__ void scale_fence() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
 template <int RT_, int DV_>
 __device__ __forceinline__ void rescale_in_place(f32x4_t (&o)[RT_][DV_], const float (&alpha)[RT_]) {
+    scale_fence();
 #pragma unroll
     for (int rt = 0; rt < RT_; ++rt)
 #pragma unroll
@@ -328,6 +333,7 @@ __device__ __forceinline__ void rescale_in_place(f32x4_t (&o)[RT_][DV_], const f
                 scale_in_place(v, alpha[rt]);
                 o[rt][j][e] = v;
             }
+    scale_fence();
 }
 
 template <int RT, bool TP>
@@ -1112,6 +1118,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     auto weighted32 = [&](int buf, const uint4 (&pf)[2], float alpha, bool rescale) {
         const uint16_t* vt = v_lds[buf];
         if (__any(rescale)) {                               // rare; in place (see scale_in_place)
+            scale_fence();
 #pragma unroll
             for (int b = 0; b < DB32; ++b)
 #pragma unroll
@@ -1120,6 +1127,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                     scale_in_place(v, alpha);
                     o32[b][i] = v;
                 }
+            scale_fence();
         }
 #pragma unroll
         for (int b = 0; b < DB32; ++b) {
