@@ -31,7 +31,15 @@ TINY_C = dict(cfg=dict(architectures=["Qwen3ForCausalLM"], vocab_size=331, hidde
                        tie_word_embeddings=True),
               block_size=4, gain_std=0.1)
 
-TINIES = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# A fourth with the head size of real checkpoints' small models (64: the kernels' 32-element
+# product steps, the wide rotation kernel) and one kv head for eight query heads.
+TINY_D = dict(cfg=dict(architectures=["Qwen3ForCausalLM"], vocab_size=500, hidden_size=128,
+                       num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=1,
+                       head_dim=64, intermediate_size=192, rms_norm_eps=1e-6, rope_theta=1e5,
+                       tie_word_embeddings=False),
+              block_size=32, gain_std=0.05)
+
+TINIES = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def write_tiny(folder, tiny, seed, dtype=torch.bfloat16, std=0.05):
