@@ -139,7 +139,8 @@ def main(argv=None):
     V = config.vocab_size
     if args.dtype == "bf16" and not args.no_tune:
         # the library's products (more than 16 rows): its fastest solution for the prompt's shapes
-        engine.tune([args.prefill_tokens] + ([] if args.no_points else [64]))
+        # and, up to 16 rows, the faster of the library and this package's own kernel for the timed batch
+        engine.tune([args.prefill_tokens] + ([] if args.no_points else [64]) + [args.batch])
 
     tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
     # bytes one decode step has to read: every weight once, and the cache of the live requests

@@ -154,16 +154,17 @@ class Engine:
     def tune(self, token_counts: Optional[Sequence[int]] = None) -> None:
         """Before serving: run a throwaway prompt of each of these lengths with the library
         timing its solutions for the model's products at that many rows (about a second per
-        shape), and keep the fastest. Default: a full portion, and the largest batch if the
-        library serves it (more than 16 rows). Steps with other numbers of rows are not
-        affected. Decode graphs are captured afterwards, so they replay the kept choices."""
+        shape), and keep the fastest; up to 16 rows, where this package's own kernel is the
+        rule, both are timed and the faster is kept for that shape. Default: a full portion,
+        and the largest batch. Steps with other numbers of rows are not affected. Decode
+        graphs are captured afterwards, so they replay the kept choices."""
         if not self.scheduler.idle:
             raise RuntimeError("tune() runs on an idle engine")
         ops = self.runner.ops
         if not hasattr(ops, "library_tuning"):
             return
         if token_counts is None:
-            token_counts = [self.scheduler.token_budget] + ([self.max_batch] if self.max_batch > 16 else [])
+            token_counts = [self.scheduler.token_budget, self.max_batch]
         kept = (self.n_steps, self.prompt_tokens, self.output_tokens)
         ops.library_tuning(True)
         try:
@@ -173,6 +174,11 @@ class Engine:
                             sampling=SamplingParams(max_new_tokens=1, eos_token_ids=()))
                 self.run()
                 self.scheduler.retire_finished()
+                if n <= 64 and ops.dtype == torch.bfloat16:
+                    # a prompt asks for one row of logits; a decode step of n requests for n
+                    model = self.runner.model
+                    rows = torch.zeros((n, model.embed.shape[1]), dtype=ops.dtype, device=ops.device)
+                    ops.linear(rows, model.head, out_dtype=torch.float32)
         finally:
             ops.library_tuning(False)
         self.n_steps, self.prompt_tokens, self.output_tokens = kept

@@ -86,6 +86,10 @@ class HipKernels:
         self.attention_splits = None        # (split_len, n_splits) override, for tests and capture
         self.attention_row_tiles = None     # row tiles per wave of the MFMA kernel, override
         self.last_attention_kernel = None   # (kernel, row tiles) the last bfloat16 call went to
+        # (rows, N, K, out dtype, partial sums welcome) -> "own" | "library" for bfloat16 products
+        # of at most 16 rows; filled while ``library_tuning`` is on, by timing both
+        self.product_choice = {}
+        self._tuning = False
         self.attention_mfma = True          # bfloat16 takes the MFMA kernels
         self.attention_workgroup = True     # prompt portions take the kernel that shares K/V through LDS
         # bfloat16 products with more than 16 rows go to the library (hipBLASLt through
@@ -215,6 +219,30 @@ class HipKernels:
             tunable.set_max_tuning_duration(30)          # ms per solution
             tunable.set_max_tuning_iterations(20)
         tunable.tuning_enable(bool(on))
+        self._tuning = bool(on)
+        if not on:
+            self._cold = None                            # the buffer that cools the caches between timed calls
+
+    def _faster(self, own, library) -> str:
+        """Time the two ways of one product and name the faster. Weights come from memory in a
+        decode step (each is read once per step, behind gigabytes of others), so a write over
+        a buffer larger than the caches comes before every timed call."""
+        if getattr(self, "_cold", None) is None:
+            self._cold = torch.empty(160 << 20, dtype=torch.float32, device=self.device)     # 640 MB
+        times = []
+        for fn in (library, own):                        # the library first: its own tuning happens at its first call
+            fn()
+            total = 0.0
+            for _ in range(6):
+                self._cold.zero_()
+                start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                fn()
+                end.record()
+                end.synchronize()
+                total += start.elapsed_time(end)
+            times.append(total)
+        return "library" if times[0] < 0.97 * times[1] else "own"
 
     def linear(self, x, w, out_dtype=None, allow_partial=False, row_tiles=0, n_waves=0, k_splits=0):
         """x [M, K] times w [N, K] transposed. float32 operands (either) take the plain
@@ -235,7 +263,24 @@ class HipKernels:
             return torch.empty((M, N), dtype=out_dtype, device=self.device)
         both_bf16 = x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
         skinny_rows = 16 if self.library_gemm else 64
-        if both_bf16 and K % 8 == 0 and K >= 8 and M <= skinny_rows:
+        own = both_bf16 and K % 8 == 0 and K >= 8 and M <= skinny_rows
+        if own and self.library_gemm and not (row_tiles or n_waves or k_splits):
+            # Up to 16 rows the skinny kernel is the rule; where a tuning pass has timed both
+            # for this shape and the library won (its kernels do not pay for the rows of x as
+            # the skinny kernel does), the library it is. Partial sums welcome: one float32 sum.
+            key = (M, N, K, out_dtype, bool(allow_partial))
+            choice = self.product_choice.get(key)
+            lib_dtype = torch.float32 if allow_partial else out_dtype
+            by_library = (lambda: torch.mm(x, w.t()) if lib_dtype == torch.bfloat16
+                          else torch.mm(x, w.t(), out_dtype=lib_dtype))
+            if choice is None and self._tuning and not torch.cuda.is_current_stream_capturing():
+                choice = self.product_choice[key] = self._faster(
+                    lambda: self.linear(x, w, out_dtype, allow_partial, -1), by_library)
+            if choice == "library":
+                out = by_library()
+                return out.unsqueeze(0) if allow_partial else out
+        row_tiles = max(row_tiles, 0)                     # -1: the skinny kernel, whatever the table says
+        if own:
             if not (row_tiles and n_waves and k_splits):
                 rw, nw, ks = c_int(0), c_int(0), c_int(0)
                 self._gemm.soc_gemm_skinny_plan(c_int(M), c_int(N), c_int(K), c_int(1 if allow_partial else 0),

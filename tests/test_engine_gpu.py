@@ -95,6 +95,19 @@ def test_tuned_library_products_leave_the_tokens_alone(tmp_path):
         engine.tune()
     engine.run()
     assert set(os.listdir(".")) == before
+    # up to 16 rows both ways of a product are timed and the faster is noted per shape; the
+    # tokens are the same whichever way the table points
+    ops = engine.runner.ops
+    engine.tune([2])
+    two_rows = [k for k in ops.product_choice if k[0] == 2]
+    assert len(two_rows) >= 4 and set(ops.product_choice.values()) <= {"own", "library"}
+    for way in ("library", "own"):
+        ops.product_choice = {k: way for k in ops.product_choice}
+        engine.runner._graphs = {}                       # captured steps hold the way they were captured with
+        got = engine.generate(prompts[:2])
+        for p, g, x in zip(prompts, got, want):
+            if margins_ok(cfg, w, p, x, 0.05):
+                assert g == x
 
 
 def test_command_line(tmp_path):
