@@ -122,3 +122,55 @@ def test_captured_decode_steps_follow_the_data(folders, oracle, dtype):
     ref = replay(eager, steps)
     for rid in ref:
         torch.testing.assert_close(got[rid], ref[rid], **TOL[dtype])
+
+
+def test_long_portion_beside_decoded_tokens_at_middle_size(tmp_path):
+    """A step of a size at which the kernels for long prompts are chosen by themselves: a
+    portion of 2,100 tokens (the eight-wave workgroup attention form, a wave per token in the
+    rotation kernel, library products) beside one decoded token of three other requests (the
+    per-wave attention kernel with key splits, in the same step), then shorter portions
+    behind that context. Head size 64, eight query heads per kv head, bfloat16."""
+    from socrates_amd.config import Qwen3Config
+    from socrates_amd.kernels import HipKernels
+    from socrates_amd.weights import write_random_model
+    cfg = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1000, hidden_size=256, num_hidden_layers=2,
+               num_attention_heads=16, num_key_value_heads=2, head_dim=64, intermediate_size=512,
+               rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True)
+    folder = write_random_model(tmp_path / "mid", Qwen3Config.from_dict(cfg), 11, dtype=torch.bfloat16, std=0.05, gain_std=0.05)
+    pcfg, w = plain.read_folder(folder)
+    prompts = random_prompts([2300, 300, 700, 40], pcfg["vocab_size"], seed=4)
+    hip = HipKernels(torch.bfloat16, DEV)
+    runner = make_runner(folder, hip, max_rows=4, max_len=2304, block_size=16)
+    cuts = [2100, 184, 16]
+    steps = [([(f"r{i}", prompts[i][:-len(cuts)], [])], []) for i in (1, 2, 3)]
+    t = 0
+    kernels = []
+    got = {}
+    rows = {}
+    from socrates_amd.engine import StepEntry
+    for entries, _ in steps:
+        rid, toks, want = entries[0]
+        rows[rid] = runner.cache.open_row()
+        runner.step([StepEntry(rows[rid], toks, want)])
+    rows["r0"] = runner.cache.open_row()
+    long_want = {}
+    for j, n in enumerate(cuts):
+        want_here = sorted({0, n // 3, n - 1})
+        batch = [StepEntry(rows[f"r{i}"], [prompts[i][len(prompts[i]) - len(cuts) + j]], [0]) for i in (1, 2, 3)]
+        batch.insert(1, StepEntry(rows["r0"], prompts[0][t:t + n], want_here))
+        logits = runner.step(batch).float().cpu()
+        kernels.append(hip.last_attention_kernel)
+        got[("r1", j)] = logits[0]
+        for a, p in enumerate(want_here):
+            long_want[t + p] = logits[1 + a]
+        got[("r2", j)], got[("r3", j)] = logits[1 + len(want_here)], logits[2 + len(want_here)]
+        t += n
+    assert kernels[0] == ("workgroup", 64) and kernels[1][0] == "wave"
+    tol = TOL[torch.bfloat16]
+    ref = plain.forward(pcfg, w, prompts[0])
+    for p, row in long_want.items():
+        torch.testing.assert_close(row, ref[p], **tol)
+    for i in (1, 2, 3):
+        ref = plain.forward(pcfg, w, prompts[i])
+        for j in range(len(cuts)):
+            torch.testing.assert_close(got[(f"r{i}", j)], ref[len(prompts[i]) - len(cuts) + j], **tol)
