@@ -27,7 +27,7 @@ class BlockAllocator:
 
     def __init__(self, num_blocks: int):
         if num_blocks < 1:
-            raise ValueError("need at least one usable block")
+            raise ValueError(f"a pool of {num_blocks} pages holds nothing: it needs one page or more")
         self.num_blocks = num_blocks
         self._stack = list(range(num_blocks, 0, -1))     # top of the stack is the end
         self._held = bytearray(num_blocks + 1)            # 1 where a page is handed out
@@ -45,9 +45,9 @@ class BlockAllocator:
 
     def alloc(self, n: int) -> list:
         if n < 0:
-            raise ValueError(f"cannot allocate {n} blocks")
+            raise ValueError(f"a request for {n} pages makes no sense")
         if n > len(self._stack):
-            raise OutOfBlocks(f"asked for {n} blocks, {len(self._stack)} free")
+            raise OutOfBlocks(f"{n} pages wanted, the pool has {len(self._stack)} left")
         if n == 0:
             return []
         pages = self._stack[-n:][::-1]
@@ -61,9 +61,9 @@ class BlockAllocator:
         seen = set()
         for p in pages:
             if p == NULL_PAGE:
-                raise ValueError("block 0 is the null page and is never allocated")
+                raise ValueError("page 0 is the null page: nobody holds it, so it cannot be given back")
             if not (0 < p <= self.num_blocks) or not self._held[p] or p in seen:
-                raise ValueError(f"block {p} freed twice, or never allocated")
+                raise ValueError(f"page {p} is not held: given back already, listed twice, or never handed out")
             seen.add(p)
         for p in pages:
             self._held[p] = 0

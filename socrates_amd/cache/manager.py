@@ -26,6 +26,7 @@ import torch
 
 from ..parts.registry import PagedKV, RowState
 from .allocator import NULL_PAGE, BlockAllocator, OutOfBlocks, blocks_for
+from .staging import PinnedUploader
 
 
 @dataclass
@@ -61,6 +62,7 @@ class PagedGroup:
         self.pool_shape = (num_blocks + 1, need.n_kv_heads, block_size, need.head_dim)
         self.dtype, self.device = dtype, device
         self.pools = {}
+        self._upload = PinnedUploader(device) if torch.device(device).type == "cuda" else None
 
     def add_slot(self, slot_id: int):
         k = torch.zeros(self.pool_shape, dtype=self.dtype, device=self.device)
@@ -113,7 +115,12 @@ class PagedGroup:
     def sync(self):
         if self.dirty:
             lo, hi = min(self.dirty), max(self.dirty) + 1
-            self.table[lo:hi].copy_(torch.from_numpy(self.host_table[lo:hi]))
+            if self._upload is not None:
+                # a snapshot in pinned memory: the host may change its table again before
+                # the queued copy runs
+                self._upload(self.host_table[lo:hi], into=self.table[lo:hi])
+            else:
+                self.table[lo:hi].copy_(torch.from_numpy(self.host_table[lo:hi]))
             self.dirty.clear()
 
 

@@ -113,6 +113,17 @@ class Qwen3Config:
             out["eos_token_id"] = eos[0] if len(eos) == 1 else list(eos)
         return out
 
+    # ---- text prompts -------------------------------------------------------------------
+    @staticmethod
+    def chat_prompt(tok, text: str):
+        """Token ids of one user turn in this architecture's chat format, as the reference
+        submits text (model/inference_paged.py:139-143): the tokenizer's chat template with the
+        generation prompt added and the model's thinking mode off."""
+        rendered = tok.apply_chat_template([{"role": "user", "content": text}], tokenize=False,
+                                           add_generation_prompt=True, enable_thinking=False)
+        ids = tok(rendered).input_ids
+        return [int(t) for t in (ids[0] if ids and isinstance(ids[0], (list, tuple)) else ids)]
+
     # ---- the layer recipe -------------------------------------------------------------
     def plan(self) -> ModelPlan:
         """Pre-norm decoder blocks, every layer alike (model/qwen/qwen_kv_paged.py:178-200)."""

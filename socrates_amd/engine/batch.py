@@ -14,6 +14,8 @@ from typing import List, Sequence
 import numpy as np
 import torch
 
+from ..cache.staging import PinnedUploader, pageable_upload  # noqa: F401
+
 
 @dataclass
 class StepEntry:
@@ -24,8 +26,21 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
+class NoHostView(dict):
+    """``StepContext.host`` of a step that is being captured into, or replayed from, a HIP
+    graph: which rows, positions and lengths the step has is then known on the device only,
+    so there is nothing to look up here. A part that walks the host arrays declares
+    ``capturable = False`` and its model's steps stay eager."""
+
+    def __missing__(self, key):
+        raise KeyError(f"ctx.host[{key!r}]: a captured step has no host-side view of its batch; a part "
+                       "that needs one declares `capturable = False`")
+
+
 @dataclass
 class StepContext:
+    """``host``: numpy copies of positions, token_rows, seq_rows, seq_qstart and seq_ctx for
+    parts that plan on the host (empty, a ``NoHostView``, in a captured step)."""
     n_tokens: int
     n_seqs: int
     n_want: int
@@ -39,10 +54,13 @@ class StepContext:
     max_q_len: int
     max_ctx_len: int
     host: dict = field(default_factory=dict)
+    upload: object = None        # int32 numpy array -> device tensor, for kernels that plan on the host
 
 
-def build_context(entries: List[StepEntry], starts: Sequence[int], device, vocab_size=None) -> StepContext:
-    """``starts[i]`` is the position of the first token of ``entries[i]``."""
+def build_context(entries: List[StepEntry], starts: Sequence[int], device, vocab_size=None,
+                  upload=None) -> StepContext:
+    """``starts[i]`` is the position of the first token of ``entries[i]``. ``upload`` brings
+    the step's integers to the device (default: a plain copy from pageable memory)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     lens = [len(e.tokens) for e in entries]
@@ -80,7 +98,8 @@ def build_context(entries: List[StepEntry], starts: Sequence[int], device, vocab
             w += 1
         t += n
     qst[S] = N
-    dev = torch.from_numpy(buf).to(device)
+    upload = upload or pageable_upload(device)
+    dev = upload(buf)
     o = 0
     views = []
     for n in (N, N, N, S, S + 1, S, n_want):
@@ -91,4 +110,4 @@ def build_context(entries: List[StepEntry], starts: Sequence[int], device, vocab
         token_rows=views[2], seq_rows=views[3], seq_qstart=views[4], seq_ctx=views[5],
         want_index=views[6], max_q_len=max(lens), max_ctx_len=int(sctx.max()),
         host={"positions": pos.copy(), "token_rows": trow.copy(), "seq_rows": srow.copy(),
-              "seq_qstart": qst.copy(), "seq_ctx": sctx.copy()})
+              "seq_qstart": qst.copy(), "seq_ctx": sctx.copy()}, upload=upload)

@@ -35,13 +35,15 @@ class Engine:
                  compile: bool = True, max_batch: int = MAX_BATCH, max_len: int = MAX_LEN,
                  max_new_tokens: int = MAX_NEW_TOKENS, block_size: int = KV_BLOCK,
                  num_blocks: Optional[int] = None, chunk: int = PREFILL_CHUNK,
-                 max_queue: int = MAX_QUEUE):
+                 max_queue: int = MAX_QUEUE, template=None):
         """model: a model folder (config.json + safetensors) or a ModelRunner. tok: an
         optional tokenizer with the HF surface the reference uses (``apply_chat_template``,
         ``__call__``, ``all_special_ids``); without one, prompts are token id lists.
         compile: replay decode-only steps from captured HIP graphs. num_blocks: pages in the
         pool; default is the worst case max_batch * ceil(max_len / block_size)
-        (model/inference_paged.py:83-84)."""
+        (model/inference_paged.py:83-84). template: ``template(tok, text) -> token ids`` for
+        text prompts; default: what the model's configuration class offers as
+        ``chat_prompt`` (the architecture's chat format), else the tokenizer's plain encoding."""
         self.device, self.max_batch = device, max_batch
         self.max_len, self.max_new_tokens = max_len, max_new_tokens
         self.tok = tok
@@ -53,9 +55,10 @@ class Engine:
                 model, dtype, device, max_rows=max_batch, max_len=max_len, block_size=block_size,
                 num_blocks=num_blocks or max_batch * per_row)
         self.cache = self.runner.cache
+        self.template = template or getattr(getattr(self.runner, "config", None), "chat_prompt", None)
         self.plan_ = self.runner.model.plan
         self.scheduler = Scheduler(self.cache, max_batch, max_len, chunk, max_queue)
-        self.sampler = Sampler(self.runner.ops, self.cache.scalars)
+        self.sampler = Sampler(self.runner.ops, self.cache.scalars, getattr(self.runner, "_upload", None))
         self.compile = compile
         if compile and hasattr(self.runner, "enable_graphs"):
             self.runner.enable_graphs(max_batch)
@@ -84,11 +87,10 @@ class Engine:
         if isinstance(prompt, str):
             if self.tok is None:
                 raise ValueError("a text prompt needs a tokenizer; pass token ids instead")
-            text = self.tok.apply_chat_template(
-                [{"role": "user", "content": prompt}], tokenize=False, add_generation_prompt=True,
-                enable_thinking=False)
-            ids = self.tok(text, return_tensors="pt").input_ids
-            ids = [int(t) for t in (ids[0].tolist() if hasattr(ids, "shape") else ids[0])]
+            if self.template is not None:
+                ids = [int(t) for t in self.template(self.tok, prompt)]
+            else:
+                ids = [int(t) for t in self.tok(prompt).input_ids]
         else:
             ids = [int(t) for t in prompt]
         eos = sampling.eos_token_ids
@@ -151,6 +153,18 @@ class Engine:
             if self.step() == 0 and not self.scheduler.idle:
                 raise RuntimeError("requests are waiting but nothing can be scheduled")
 
+    def warmup(self, max_width: Optional[int] = None, max_context: Optional[int] = None) -> int:
+        """Before serving: capture the decode graphs of every width bucket up to
+        ``max_width`` (default ``max_batch``) and every context bucket up to ``max_context``
+        (default ``max_len``), as the reference does when its engine is built
+        (model/inference_paged.py:110-130); without it a graph is captured at the first step
+        that needs it. Returns the number of graphs held (0: steps are not captured)."""
+        if not self.scheduler.idle:
+            raise RuntimeError("warmup() runs on an idle engine")
+        if not hasattr(self.runner, "warmup"):
+            return 0
+        return self.runner.warmup(max_width or self.max_batch, max_context or self.max_len)
+
     def tune(self, token_counts: Optional[Sequence[int]] = None) -> None:
         """Before serving: run a throwaway prompt of each of these lengths with the library
         timing its solutions for the model's products at that many rows (about a second per
@@ -176,9 +190,8 @@ class Engine:
                 self.scheduler.retire_finished()
                 if n <= 64 and ops.dtype == torch.bfloat16:
                     # a prompt asks for one row of logits; a decode step of n requests for n
-                    model = self.runner.model
-                    rows = torch.zeros((n, model.embed.shape[1]), dtype=ops.dtype, device=ops.device)
-                    ops.linear(rows, model.head, out_dtype=torch.float32)
+                    self.runner.model.head_logits(torch.zeros(
+                        (n, self.plan_.hidden), dtype=ops.dtype, device=ops.device))
         finally:
             ops.library_tuning(False)
         self.n_steps, self.prompt_tokens, self.output_tokens = kept

@@ -3,7 +3,10 @@
 Names and meanings are the reference's (model/inference_cont.py:21-24, 36-40,
 65-82): MAX_BATCH rows, MAX_NEW_TOKENS per request, MAX_LEN slots per row,
 MAX_QUEUE waiting requests; ``QueueFull`` and ``TooLong``; a ``Request`` with its
-ids, output, row and timestamps.
+ids, output, row and timestamps. The values are not the reference's, which are sized
+for a 24 GB GPU (18 rows of 2,048 slots): here 64 rows of 4,096 slots, whose worst-case
+page pool is 39 GB at Qwen3-4B sizes and 69 GB at Qwen3-32B sizes, beside the weights
+in 288 GB.
 """
 
 from __future__ import annotations
@@ -15,9 +18,9 @@ from typing import List, Optional
 
 from ..sampling import SamplingParams
 
-MAX_BATCH = 18
+MAX_BATCH = 64
 MAX_NEW_TOKENS = 1024
-MAX_LEN = 2048
+MAX_LEN = 4096
 MAX_QUEUE = 16 * MAX_BATCH
 
 

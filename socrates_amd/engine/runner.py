@@ -17,7 +17,7 @@ from ..cache import CacheManager
 from ..config import load_config
 from ..parts import DecoderModel, cache_needs, expected_tensors
 from ..weights import load_weights
-from .batch import StepContext, StepEntry, build_context
+from .batch import NoHostView, PinnedUploader, StepContext, StepEntry, build_context
 
 
 class ModelRunner:
@@ -25,9 +25,13 @@ class ModelRunner:
         self.model, self.cache = model, cache
         self.ops = model.ops
         self.vocab_size = model.plan.vocab_size
-        self._graphs = None              # width -> captured decode step, once enable_graphs ran
+        self._graphs = None              # (width, context) -> captured decode step, once enable_graphs ran
         self._staging_read = {}          # per captured step: event behind the last copy out of its staging buffer
         self._graph_max = 0
+        self._graph_pool = None          # one memory pool for all captures: replays never overlap
+        self.graphs_refused = None       # why enable_graphs left the steps eager, if it did
+        # eager steps: the batch's integers go through pinned staging memory, one copy per step
+        self._upload = PinnedUploader(self.ops.device) if self.ops.device.type == "cuda" else None
 
     @classmethod
     def from_folder(cls, folder, dtype, device, max_rows, max_len, block_size, num_blocks, ops=None):
@@ -59,7 +63,7 @@ class ModelRunner:
                 and all(len(e.tokens) == 1 for e in entries)):
             return self._step_captured(entries, borrow)
         starts = [cache.length(e.row) for e in entries]
-        ctx = build_context(entries, starts, self.ops.device, self.vocab_size)
+        ctx = build_context(entries, starts, self.ops.device, self.vocab_size, self._upload)
         for e, start in zip(entries, starts):
             cache.reserve(e.row, start + len(e.tokens))
         cache.sync()
@@ -79,10 +83,18 @@ class ModelRunner:
     _BUCKETS = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 
     def enable_graphs(self, max_width: int) -> None:
+        """From now on steps in which every request brings one token are replayed from HIP
+        graphs, up to ``max_width`` requests. A model with a part that cannot be captured
+        (``capturable = False``: it reads the host's view of the batch or waits for the
+        device) keeps all its steps eager; ``graphs_refused`` then says so."""
         if self.ops.device.type != "cuda":
             return                       # a stand-in kernel set on the CPU has nothing to capture
+        if not getattr(self.model, "capturable", True):
+            self.graphs_refused = "a part of the model declares capturable = False"
+            return
         self._graphs = {}
         self._graph_max = max_width
+        self._graph_pool = torch.cuda.graph_pool_handle()
 
     def _bucket(self, n: int) -> int:
         for b in self._BUCKETS:
@@ -98,16 +110,42 @@ class ModelRunner:
             b *= 2
         return min(b, self.cache.max_len)
 
+    def warmup(self, max_width: int = None, max_context: int = None) -> int:
+        """Capture, before serving, the decode step of every width bucket up to ``max_width``
+        (default: what enable_graphs was given) for every context bucket up to
+        ``max_context`` (default: the cache's longest row), as the reference captures all
+        its widths when the engine is built (model/inference_paged.py:110-130). Returns the
+        number of graphs now held. All captures share one memory pool (replays never
+        overlap), so what they hold beyond it is one float32 logits buffer [width, vocab]
+        per graph."""
+        if self._graphs is None:
+            return 0
+        max_width = min(max_width or self._graph_max, self._graph_max)
+        contexts, c = [], 256
+        longest = min(max_context or self.cache.max_len, self.cache.max_len)
+        while True:
+            contexts.append(min(c, self.cache.max_len))
+            if c >= longest:
+                break
+            c *= 2
+        widths = sorted({self._bucket(n) for n in range(1, max_width + 1)})
+        for context in sorted(set(contexts)):
+            for width in widths:
+                if (width, context) not in self._graphs:
+                    self._graphs[(width, context)] = self._capture(width, context)
+        return len(self._graphs)
+
     def _capture(self, width: int, context: int):
         dev = self.ops.device
-        inputs = torch.zeros((3, width), dtype=torch.int32, device=dev)
+        # rows of the input buffer: token ids, positions, cache rows, lengths after the step
+        inputs = torch.zeros((4, width), dtype=torch.int32, device=dev)
         inputs[2].fill_(self.cache.null_row)
-        staging = torch.zeros((3, width), dtype=torch.int32).pin_memory()
+        staging = torch.zeros((4, width), dtype=torch.int32).pin_memory()
         arange = torch.arange(width + 1, dtype=torch.int32, device=dev)
         ctx = StepContext(
             n_tokens=width, n_seqs=width, n_want=width, token_ids=inputs[0], positions=inputs[1],
-            token_rows=inputs[2], seq_rows=inputs[2], seq_qstart=arange, seq_ctx=inputs[1],
-            want_index=arange[:width], max_q_len=1, max_ctx_len=context, host={})
+            token_rows=inputs[2], seq_rows=inputs[2], seq_qstart=arange, seq_ctx=inputs[3],
+            want_index=arange[:width], max_q_len=1, max_ctx_len=context, host=NoHostView())
         stream = torch.cuda.Stream(device=dev)
         stream.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(stream):
@@ -115,7 +153,7 @@ class ModelRunner:
         torch.cuda.current_stream(dev).wait_stream(stream)
         torch.cuda.synchronize(dev)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
+        with torch.cuda.graph(graph, pool=self._graph_pool, stream=stream):
             logits = self.model.forward(ctx, self.cache)
         # The graph holds raw addresses: every tensor it reads (the inputs, and ``arange``
         # through ctx) has to live as long as the graph, so ctx is kept beside it.
@@ -139,7 +177,7 @@ class ModelRunner:
         if copied is not None:
             copied.synchronize()            # the last step's copy has read the staging buffer
         host = staging.numpy()
-        host[0, n:], host[1, n:], host[2, n:] = 0, 0, cache.null_row
+        host[0, n:], host[1, n:], host[2, n:], host[3, n:] = 0, 0, cache.null_row, 0
         for i, e in enumerate(entries):
             token = int(e.tokens[0])
             if not 0 <= token < self.vocab_size:
@@ -148,7 +186,7 @@ class ModelRunner:
                 raise ValueError(f"entry {i}: wanted place outside its one token")
             start = cache.length(e.row)
             cache.reserve(e.row, start + 1)
-            host[0, i], host[1, i], host[2, i] = token, start, e.row
+            host[0, i], host[1, i], host[2, i], host[3, i] = token, start, e.row, start + 1
         cache.sync()
         inputs.copy_(staging, non_blocking=True)
         copied = copied or torch.cuda.Event()

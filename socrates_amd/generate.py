@@ -97,16 +97,17 @@ def main(argv=None) -> int:
     reqs = [engine.submit(p, sampling=SamplingParams(
         temperature=args.temperature, seed=args.seed + i,
         eos_token_ids=None if args.eos is None else tuple(args.eos))) for i, p in enumerate(prompts)]
-    print(f"{len(reqs)} requests, {engine.max_batch} rows, "
-          f"{engine.cache.groups[0].allocator.num_blocks} blocks of {engine.cache.block_size}\n")
+    pools = ", ".join(f"{g.allocator.num_blocks} pages of {g.block_size} tokens" for g in engine.cache.groups)
+    print(f"{len(reqs)} requests, {engine.max_batch} rows, {pools or 'no paged cache'}\n")
     t0 = time.perf_counter()
     engine.run()
     wall = time.perf_counter() - t0
     for r in reqs:
         shown = tok.decode(r.output) if tok is not None else " ".join(map(str, r.output))
-        print(f"> {r.prompt if isinstance(r.prompt, str) else ' '.join(map(str, r.ids))}\n{shown}\n")
+        asked = r.prompt if isinstance(r.prompt, str) else " ".join(map(str, r.ids))
+        print(f"> {asked}\n{shown}\n")
     total = sum(len(r.output) for r in reqs)
-    print(f"{wall:.2f}s | {total} tok | {total / wall:.2f} tok/s")
+    print(f"{wall:.2f} s wall | {total} tok | {total / wall:.2f} tok/s")
     return 0
 
 

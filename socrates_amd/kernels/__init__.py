@@ -17,7 +17,8 @@ import torch
 
 from .build import KernelBuildError, build_all, compile_library, load_library
 
-__all__ = ["HipKernels", "KernelBuildError", "build_all", "compile_library", "load_library"]
+__all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "build_all", "compile_library",
+           "load_library", "plan_key_splits"]
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -65,6 +66,22 @@ def _declare(lib, signatures):
     for name, argtypes in signatures.items():
         fn = getattr(lib, name)
         fn.argtypes, fn.restype = argtypes, (None if name.endswith("_plan") else c_int)
+
+
+MAX_KEY_SPLITS = 256    # what the merge kernel of the MFMA attention holds weights for
+
+
+def plan_key_splits(n_blocks, n_kv_heads, group, max_keys):
+    """(split_len, n_splits) for the MFMA attention kernel: enough waves to fill the GPU, no
+    split shorter than 64 keys, at most MAX_KEY_SPLITS of them (a longer context gets longer
+    splits). Splits are over absolute key indices, a multiple of 16 keys long, and cover keys
+    0 .. max_keys - 1. Host arithmetic only."""
+    waves = n_blocks * n_kv_heads * ((group + 15) // 16)
+    # from one wave per SIMD on (1,024) no split: the merge costs a wave per (token, head)
+    n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64,
+                                           MAX_KEY_SPLITS))
+    split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
+    return split_len, (max_keys + split_len - 1) // split_len
 
 
 class HipKernels:
@@ -439,21 +456,23 @@ class HipKernels:
             first = qstart[seq] + j * tokens_per_block
             n = np.minimum(tokens_per_block, lens[seq] - j * tokens_per_block)
             blocks = np.stack([first, n], 1).astype(np.int32)
-            cache[key] = (torch.from_numpy(blocks).to(self.device), len(blocks))
+            upload = getattr(ctx, "upload", None)
+            dev = upload(blocks) if upload is not None else torch.from_numpy(blocks).to(self.device)
+            cache[key] = (dev, len(blocks))
         return cache[key]
 
     def plan_mfma(self, n_blocks, n_kv_heads, group, max_keys):
-        """(split_len, n_splits) for the MFMA kernel: enough waves to fill the GPU, no split
-        shorter than 64 keys. Splits are over absolute key indices."""
+        """(split_len, n_splits) for the MFMA kernel; an override (``attention_splits``) is
+        rounded to what the kernel takes and refused beyond its limit."""
         if self.attention_splits is not None:
             split_len, n_splits = self.attention_splits
             split_len = max(16, (min(split_len, 1 << 24) + 15) // 16 * 16)
-            return split_len, max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
-        waves = n_blocks * n_kv_heads * ((group + 15) // 16)
-        # from one wave per SIMD on (1,024) no split: the merge costs a wave per (token, head)
-        n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64))
-        split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
-        return split_len, (max_keys + split_len - 1) // split_len
+            n_splits = max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
+            if n_splits > MAX_KEY_SPLITS:
+                raise KernelError(f"{n_splits} key splits asked for; the MFMA attention kernel merges at "
+                                  f"most {MAX_KEY_SPLITS}")
+            return split_len, n_splits
+        return plan_key_splits(n_blocks, n_kv_heads, group, max_keys)
 
     def _wave_attention(self, lib, q, slot, ctx, out, scale, w, rt, gpl, which):
         """The per-wave MFMA kernel with key splits and merge, for all sequences of the step

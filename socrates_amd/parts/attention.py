@@ -48,6 +48,7 @@ class PagedAttention:
         self.eps = spec.qk_norm.eps if spec.qk_norm is not None else 0.0
         self.position = (build_part(spec.position, {}, ops)
                          if spec.position is not None else None)
+        self.capturable = getattr(self.position, "capturable", True)
 
     def forward(self, x, ctx, slot, write=True):
         s, ops = self.spec, self.ops

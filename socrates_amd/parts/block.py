@@ -50,6 +50,10 @@ class PreNormBlock:
         self.mixer = build_part(spec.mixer, _sub_tensors(spec, "mixer", weights), ops)
         self.norm2 = build_part(spec.norm2, _sub_tensors(spec, "norm2", weights), ops)
         self.ffn = build_part(spec.ffn, _sub_tensors(spec, "ffn", weights), ops)
+        # a step through this layer can be captured into a HIP graph unless one of its parts
+        # says otherwise (it reads the host's view of the batch, or syncs with the device)
+        self.capturable = all(getattr(p, "capturable", True)
+                              for p in (self.norm1, self.mixer, self.norm2, self.ffn))
 
     def forward(self, residual, pending, ctx, slot, write=True):
         """residual: fp32 [N, hidden], updated in place. pending: the previous block's

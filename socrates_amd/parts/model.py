@@ -52,6 +52,9 @@ class DecoderModel:
                         for local in tensors_of(plan.final_norm)}
         self.final_norm = build_part(plan.final_norm, norm_tensors, ops)
         self.head = self.embed if plan.head_name is None else weights[plan.head_name]
+        # False if any part declares `capturable = False`: the runner then runs every step eagerly
+        self.capturable = (all(getattr(b, "capturable", True) for b in self.blocks)
+                           and getattr(self.final_norm, "capturable", True))
 
     def forward(self, ctx, cache):
         """ctx: a StepContext on the device; cache: the CacheManager. Returns float32
@@ -66,4 +69,8 @@ class DecoderModel:
             # The cache is complete after the last block; no logits are asked for.
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=ops.device)
         h = self.final_norm.add_norm(residual, pending, rows=ctx.want_index)
-        return ops.linear(h, self.head, out_dtype=torch.float32)
+        return self.head_logits(h)
+
+    def head_logits(self, h):
+        """float32 logits [n, vocab] of normed rows ``h`` [n, hidden]."""
+        return self.ops.linear(h, self.head, out_dtype=torch.float32)

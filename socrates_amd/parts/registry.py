@@ -20,6 +20,13 @@ Interfaces (duck-typed):
   mixer        ``cache_need(spec) -> PagedKV | RowState | None`` (staticmethod)
                ``forward(x, ctx, slot, write) -> y`` with x, y [N, hidden]
   feed-forward ``forward(x, ctx) -> y``
+
+A part whose ``forward`` reads ``ctx.host`` (the host's copy of the step's rows, positions
+and sequence starts), or waits for the device, sets ``capturable = False`` (class or
+instance attribute): a model with such a part never has its decode steps captured into HIP
+graphs, whatever the engine's ``compile`` says. Parts without the attribute are taken to
+be capturable: everything they do is device work on the current stream whose launch
+shape depends on the step only through ``ctx.n_tokens`` and ``ctx.max_ctx_len``.
 """
 
 from __future__ import annotations

@@ -34,9 +34,10 @@ class SamplingParams:
 
 
 class Sampler:
-    def __init__(self, ops, scalars):
-        """ops: the kernel set; scalars: the cache manager's RowScalars."""
-        self.ops, self.scalars = ops, scalars
+    def __init__(self, ops, scalars, upload=None):
+        """ops: the kernel set; scalars: the cache manager's RowScalars; upload: int32 numpy
+        array -> device tensor (the step function's pinned staging), default a plain copy."""
+        self.ops, self.scalars, self.upload = ops, scalars, upload
 
     def sample(self, logits: torch.Tensor, rows: Sequence[int]):
         """One token for each row of ``logits`` (float32 [n, vocab]); ``rows[i]`` is the cache
@@ -50,10 +51,16 @@ class Sampler:
         if not temperature.any():
             tokens = self.ops.argmax(logits)
         else:
-            dev = logits.device
-            tokens = self.ops.sample(
-                logits, torch.from_numpy(temperature).to(dev),
-                torch.from_numpy(self.scalars.seed[idx].astype(np.int64)).to(dev),
-                torch.from_numpy(self.scalars.draws[idx]).to(dev))
+            # one copy for the three arrays: seeds and draws (64-bit, first, so that they are
+            # aligned) and the temperatures, as 32-bit words
+            n = len(idx)
+            words = np.empty(5 * n, dtype=np.int32)
+            words[:2 * n] = self.scalars.seed[idx].astype(np.int64).view(np.int32)
+            words[2 * n:4 * n] = self.scalars.draws[idx].astype(np.int64).view(np.int32)
+            words[4 * n:] = temperature.astype(np.float32).view(np.int32)
+            dev = (self.upload(words) if self.upload is not None
+                   else torch.from_numpy(words).to(logits.device))
+            tokens = self.ops.sample(logits, dev[4 * n:].view(torch.float32),
+                                     dev[:2 * n].view(torch.int64), dev[2 * n:4 * n].view(torch.int64))
         self.scalars.draws[idx] += 1
         return [int(t) for t in tokens.tolist()]

@@ -110,18 +110,21 @@ def block(x, w, i, cfg, positions):
     return x + swiglu_mlp(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
 
 
-def forward(cfg, w, ids, first_position=0):
+def forward(cfg, w, ids, first_position=0, rows=None):
     """model/qwen/qwen_kv_paged.py:219-224: embed, blocks, final norm, logits = x E^T.
     The reference always uses the embedding table as the head (:224); a folder with
     tie_word_embeddings=false carries lm_head.weight, used instead.
 
-    ids: sequence of token ids. Returns logits [T, V] for every position.
+    ids: sequence of token ids. Returns logits [T, V] for every position, or for the
+    positions listed in ``rows`` only (a large vocabulary makes all of them costly).
     """
     ids = torch.as_tensor(ids, dtype=torch.long)
     positions = torch.arange(first_position, first_position + len(ids))
     x = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         x = block(x, w, i, cfg, positions)
+    if rows is not None:
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ head.T

@@ -13,7 +13,19 @@ from socrates_amd.config.specs import ModelPlan, RunStep
 from socrates_amd.parts import expected_tensors
 from socrates_amd.weights import WeightError, load_weights, write_random_model
 
-REFERENCE_4B = "/root/reference/model/configs/qwen3-4b.json"
+# The reference's pinned configuration of Qwen3-4B (model/configs/qwen3-4b.json), with every key it
+# carries, ignored ones included. Kept here as data so that the test runs wherever the
+# repository is checked out; SOCRATES_REFERENCE may name a checkout of the reference to
+# compare this copy with.
+REFERENCE_4B = {
+    "architectures": ["Qwen3ForCausalLM"], "attention_bias": False, "attention_dropout": 0.0,
+    "bos_token_id": 151643, "eos_token_id": 151645, "head_dim": 128, "hidden_act": "silu",
+    "hidden_size": 2560, "initializer_range": 0.02, "intermediate_size": 9728,
+    "max_position_embeddings": 40960, "max_window_layers": 36, "model_type": "qwen3",
+    "num_attention_heads": 32, "num_hidden_layers": 36, "num_key_value_heads": 8,
+    "rms_norm_eps": 1e-06, "rope_scaling": None, "rope_theta": 1000000, "sliding_window": None,
+    "tie_word_embeddings": True, "torch_dtype": "bfloat16", "transformers_version": "4.51.0",
+    "use_cache": True, "use_sliding_window": False, "vocab_size": 151936}
 
 
 def test_reads_every_size_from_its_own_keys():
@@ -36,11 +48,14 @@ def test_reads_every_size_from_its_own_keys():
     assert len(plan.layers) == 3 and [s.layer for s in plan.order] == [0, 1, 2]
 
 
-def test_reference_config_file_reads_if_present():
+def test_reference_config_reads(tmp_path):
     import os
-    if not os.path.exists(REFERENCE_4B):
-        pytest.skip("reference not mounted")
-    cfg = Qwen3Config.from_json(REFERENCE_4B)              # model/configs/qwen3-4b.json
+    (tmp_path / "config.json").write_text(json.dumps(REFERENCE_4B))
+    cfg = Qwen3Config.from_json(tmp_path)                  # model/configs/qwen3-4b.json
+    assert load_config(tmp_path) == cfg                    # through the registry too
+    checkout = os.environ.get("SOCRATES_REFERENCE")
+    if checkout:
+        assert json.loads(open(os.path.join(checkout, "model/configs/qwen3-4b.json")).read()) == REFERENCE_4B
     assert (cfg.num_hidden_layers, cfg.hidden_size, cfg.head_dim) == (36, 2560, 128)
     assert cfg.tie_word_embeddings and cfg.eos_token_ids == (151645,)
     counts = cfg.param_counts()
@@ -95,11 +110,7 @@ def test_presets_that_come_with_the_package():
     assert (a.head_dim, a.tie_word_embeddings, b.head_dim, b.tie_word_embeddings) == (16, True, 32, False)
     with pytest.raises(ConfigError, match="unknown preset.*qwen3-4b"):
         preset_path("qwen3-400b")
-    try:
-        pinned = json.loads(open(REFERENCE_4B).read())
-    except OSError:
-        return
-    ours, theirs = load_preset("qwen3-4b"), Qwen3Config.from_dict(pinned)
+    ours, theirs = load_preset("qwen3-4b"), Qwen3Config.from_dict(REFERENCE_4B)
     for key in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads",
                 "head_dim", "intermediate_size", "rms_norm_eps", "rope_theta", "tie_word_embeddings"):
         assert getattr(ours, key) == getattr(theirs, key), key

@@ -559,3 +559,34 @@ def test_attention_far_key_stands_out(kernel_sets, dtype, far):
         got = hip.paged_attention(q, slot, ctx_for([0], [n - 1]), 1.0)
         close(got.cpu(), want, dtype, atol=3e-5 if dtype == torch.float32 else 3e-2)
     hip.attention_splits = None
+
+
+@pytest.mark.parametrize("Hq,Hkv,n", [(8, 2, 20000), (16, 4, 16448), (4, 1, 33000)])
+def test_decoded_token_behind_a_long_context(kernel_sets, Hq, Hkv, n):
+    """One decoded token behind tens of thousands of keys, at head counts for which the planner
+    once asked for more key splits than the merge kernel holds (313, 257 and 512): the plan
+    stays within the limit and the result equals plain attention, with one far key made to
+    stand out so that a split that is skipped or merged wrongly shows."""
+    from socrates_amd.kernels import MAX_KEY_SPLITS, KernelError
+    hip, _ = kernel_sets[torch.bfloat16]
+    D, bs = 64, 16
+    slot, dense = make_paged_case([n], Hq, Hkv, D, bs, torch.bfloat16, seed=n)
+    far = n // 3 + 5
+    u = torch.nn.functional.normalize(torch.randn(D), dim=0)
+    q = (0.1 * torch.randn(1, Hq, D) + 4.0 * u).to(torch.bfloat16).to(DEV)
+    page, off = int(slot.block_table[0, far // bs]), far % bs
+    slot.k[page, :, off] = (4.0 * u).to(torch.bfloat16).to(DEV)
+    dense[0][0][:, far] = slot.k[page, :, off].float().cpu()
+    split_len, n_splits = hip.plan_mfma(1, Hkv, Hq // Hkv, n)
+    assert n_splits <= MAX_KEY_SPLITS and n_splits * split_len >= n
+    want = dense_attention(q, dense, [0], [n - 1], 1.0)
+    got = hip.paged_attention(q, slot, ctx_for([0], [n - 1]), 1.0)
+    assert hip.last_attention_kernel[0] == "wave"
+    close(got.cpu(), want, torch.bfloat16, atol=3e-2)
+    # an override beyond the limit is refused on the host, with the limit in the message
+    hip.attention_splits = (16, 100000)
+    try:
+        with pytest.raises(KernelError, match="at most 256"):
+            hip.paged_attention(q, slot, ctx_for([0], [n - 1]), 1.0)
+    finally:
+        hip.attention_splits = None

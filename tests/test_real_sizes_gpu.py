@@ -1,0 +1,97 @@
+"""Logits at the layer sizes the benchmark times: two layers with the widths of Qwen3-4B
+(hidden 2,560, 32 query and 8 kv heads of 128, feed-forward 9,728, vocabulary 151,936, tied
+head), seeded weights written as a folder that the plain implementation reads on the CPU.
+The reference compares every logit of its model at every step (tests/test_paged_model.py:35-76);
+here the same at real widths, where the decode products split K, the feed-forward's
+activation sits in a product's epilogue, the head has 151,936 rows and the attention kernels
+run with 32 / 8 heads of 128 and many key splits."""
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import make_runner, random_prompts
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# float32: 1e-4 of the logit scale (the reference's bound for whole-model logits); bfloat16 as
+# in the replay tests
+TOL = {torch.float32: dict(atol=4e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
+WIDE = dict(architectures=["Qwen3ForCausalLM"], vocab_size=151936, hidden_size=2560, num_hidden_layers=2,
+            num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=9728,
+            rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True)
+
+
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    from socrates_amd.config import Qwen3Config
+    from socrates_amd.weights import write_random_model
+    folder = write_random_model(tmp_path_factory.mktemp("wide") / "m", Qwen3Config.from_dict(WIDE), 21,
+                                dtype=torch.bfloat16, std=0.02, gain_std=0.1)
+    cfg, w = plain.read_folder(folder)
+    prompts = random_prompts([300, 2200, 90, 500, 33], cfg["vocab_size"], seed=5)
+    return folder, cfg, w, prompts
+
+
+def close(got, want, dtype, what):
+    tol = TOL[dtype]
+    bad = (got - want).abs() > tol["atol"] + tol["rtol"] * want.abs()
+    assert not bad.any(), (f"{what}: {int(bad.sum())} logits off, largest error "
+                           f"{float((got - want).abs().max()):.3g} at scale {float(want.abs().max()):.3g}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_whole_prompt_then_captured_decode(wide, dtype):
+    """A 300-token prompt: most of it in one step, then its last 32 tokens one by one
+    through captured graphs (one row: the skinny products with K splits, the SwiGLU epilogue,
+    the float32-output head of 151,936 rows, decode attention with key splits)."""
+    from socrates_amd.engine import StepEntry
+    from socrates_amd.kernels import HipKernels
+    folder, cfg, w, prompts = wide
+    prompt = prompts[0]
+    head_rows = [0, 1, 15, 16, 17, 100, 255, 256, 267]
+    want = plain.forward(cfg, w, prompt, rows=head_rows + list(range(268, 300)))
+    runner = make_runner(folder, HipKernels(dtype, DEV), max_rows=2, max_len=512, block_size=16)
+    runner.enable_graphs(2)
+    row = runner.cache.open_row()
+    got = runner.step([StepEntry(row, prompt[:268], head_rows)]).float().cpu()
+    close(got, want[:len(head_rows)], dtype, "the prompt's first 268 tokens in one step")
+    for t in range(268, 300):
+        logits = runner.step([StepEntry(row, prompt[t:t + 1], [0])]).float().cpu()
+        close(logits[0], want[len(head_rows) + t - 268], dtype, f"decoded token at position {t}")
+    assert list(runner._graphs) == [(1, 512)]           # every decoded token came from the one captured step
+    runner.cache.close_row(row)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_long_portion_beside_decoded_tokens(wide, dtype):
+    """A mixed step at real widths: a 2,100-token portion of one request (the eight-wave
+    attention form, library or plain products of 2,100 rows) beside one decoded token of three
+    other requests behind contexts of 89, 499 and 32 tokens, then the rest of the long request
+    in a second mixed step."""
+    from socrates_amd.engine import StepEntry
+    from socrates_amd.kernels import HipKernels
+    folder, cfg, w, prompts = wide
+    ops = HipKernels(dtype, DEV)
+    runner = make_runner(folder, ops, max_rows=4, max_len=2304, block_size=16)
+    rows = {}
+    for i in (2, 3, 4):                                   # everything but their last two tokens
+        rows[i] = runner.cache.open_row()
+        runner.step([StepEntry(rows[i], prompts[i][:-2], [])])
+    rows[1] = runner.cache.open_row()
+    long_prompt = prompts[1]
+    wanted = {1: [0, 700, 2099, 2100, 2150, 2199], 2: [88, 89], 3: [498, 499], 4: [31, 32]}
+    oracle = {i: plain.forward(cfg, w, prompts[i], rows=r) for i, r in wanted.items()}
+    cuts = [(0, 2100, [0, 700, 2099]), (2100, 100, [0, 50, 99])]
+    for j, (start, n, want_here) in enumerate(cuts):
+        batch = [StepEntry(rows[2], [prompts[2][-2 + j]], [0]),
+                 StepEntry(rows[1], long_prompt[start:start + n], want_here),
+                 StepEntry(rows[3], [prompts[3][-2 + j]], [0]),
+                 StepEntry(rows[4], [prompts[4][-2 + j]], [0])]
+        logits = runner.step(batch).float().cpu()
+        if dtype == torch.bfloat16 and j == 0:
+            assert ops.last_attention_kernel == ("workgroup", 64)   # the long portion; the short ones by key splits
+        close(logits[0], oracle[2][j], dtype, f"step {j}: decoded token of the 90-token request")
+        close(logits[1:4], oracle[1][3 * j:3 * j + 3], dtype, f"step {j}: the long portion")
+        close(logits[4], oracle[3][j], dtype, f"step {j}: decoded token of the 500-token request")
+        close(logits[5], oracle[4][j], dtype, f"step {j}: decoded token of the 33-token request")

@@ -174,3 +174,50 @@ def test_long_portion_beside_decoded_tokens_at_middle_size(tmp_path):
         ref = plain.forward(pcfg, w, prompts[i])
         for j in range(len(cuts)):
             torch.testing.assert_close(got[(f"r{i}", j)], ref[len(prompts[i]) - len(cuts) + j], **tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("name,live,longest", [("B", 5, 120), ("B", 11, 400), ("D", 23, 120), ("D", 40, 400),
+                                              ("C", 40, 300)])
+def test_captured_steps_of_padded_widths_and_long_contexts(folders, name, live, longest, dtype):
+    """Decode steps of 5, 11, 23 and 40 live rows replay the graphs of the width buckets 6,
+    12, 24 and 48 (the padding rows use the null row), with contexts inside the 256-key bucket
+    and beyond it. Every replay is compared with the plain implementation; between replays
+    there is eager work (a portion of another request) and rows leave one by one, so the same
+    graph is replayed with other rows, other lengths and more padding."""
+    import random
+    from socrates_amd.engine import StepEntry
+    tiny = TINIES[name]
+    cfg, w = plain.read_folder(folders[name])
+    rng = random.Random(live)
+    lengths = [longest] + [rng.randrange(12, longest) for _ in range(live - 1)]
+    prompts = random_prompts(lengths, cfg["vocab_size"], seed=live)
+    tail = 6
+    want = [plain.forward(cfg, w, p)[-tail:] for p in prompts]
+    from socrates_amd.kernels import HipKernels
+    runner = make_runner(folders[name], HipKernels(dtype, DEV), max_rows=live + 1, max_len=512,
+                         block_size=tiny["block_size"])
+    runner.enable_graphs(64)
+    rows = []
+    for p in prompts:
+        rows.append(runner.cache.open_row())
+        runner.step([StepEntry(rows[-1], p[:-tail], [])])
+    extra = runner.cache.open_row()
+    extra_prompt = random_prompts([40], cfg["vocab_size"], seed=99)[0]
+    extra_want = plain.forward(cfg, w, extra_prompt)
+    alive = list(range(live))
+    for t in range(tail):
+        batch = [StepEntry(rows[i], [prompts[i][len(prompts[i]) - tail + t]], [0]) for i in alive]
+        logits = runner.step(batch).float().cpu()
+        for j, i in enumerate(alive):
+            torch.testing.assert_close(logits[j], want[i][t], **TOL[dtype],
+                                       msg=lambda m: f"step {t}, request {i} of {len(alive)} live: {m}")
+        # eager work between the replays: a portion of another request, checked as well
+        got = runner.step([StepEntry(extra, extra_prompt[6 * t:6 * t + 6], [5])]).float().cpu()
+        torch.testing.assert_close(got[0], extra_want[6 * t + 5], **TOL[dtype])
+        if t >= 2 and len(alive) > 2:
+            runner.cache.close_row(rows[alive.pop(1)])    # a row leaves: same bucket, one more padding row
+    widths = {k[0] for k in runner._graphs}
+    contexts = {k[1] for k in runner._graphs}
+    assert runner._bucket(live) in widths and runner._bucket(live) >= live
+    assert (512 in contexts) == (longest > 256), (contexts, longest)

@@ -237,6 +237,8 @@ class DecaySpec:
 
 
 class DecayMixer:
+    capturable = False          # walks the host's view of the batch: its steps must stay eager
+
     @staticmethod
     def tensors(spec):
         return {"mix.weight": TensorDecl((spec.hidden, spec.hidden))}
@@ -298,6 +300,44 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(kind, dtype):
     torch.testing.assert_close(whole, want, **tol)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_a_model_with_a_stateful_toy_mixer_generates_through_the_engine(dtype):
+    """``Engine(compile=True)``, the default, with a model one of whose parts cannot be
+    captured: the runner keeps every step eager (and says why), generation works, tokens are
+    those of ``compile=False``, and a model of capturable parts beside it does get its graphs.
+    A captured step's context has no host view, and says so when asked."""
+    from socrates_amd.engine import Engine, NoHostView
+    from socrates_amd.kernels import HipKernels
+    register_part(DecaySpec, DecayMixer)
+    ops = HipKernels(dtype, "cuda:0")
+    hidden = 32
+    toy = BlockSpec(DecaySpec(hidden, 0.9), SwiGLUSpec(hidden, 40), RMSNormSpec(hidden, 1e-5),
+                    RMSNormSpec(hidden, 1e-5), prefix="model.layers.1.",
+                    names=(("norm1", "n1"), ("mixer", "decay"), ("norm2", "n2"), ("ffn", "mlp")))
+    prompts = random_prompts([9, 3, 14], 50, seed=2)
+    outs = {}
+    for label, layers, compile_ in (("toy", [qwen_like_block(0), toy], True), ("toy-eager", [qwen_like_block(0), toy], False),
+                                    ("plain", [qwen_like_block(0), qwen_like_block(1)], True)):
+        plan = plan_with(layers, [RunStep(0, 0), RunStep(1, 1)], hidden)
+        weights = random_tensors(expected_tensors(plan), seed=3, dtype=dtype, device="cuda:0", std=0.2, gain_std=0.1)
+        model = DecoderModel(plan, weights, ops)
+        cache = CacheManager(cache_needs(plan), 4, 64, 8, 32, dtype, "cuda:0")
+        engine = Engine(ModelRunner(model, cache), max_batch=4, max_len=64, max_new_tokens=10, compile=compile_)
+        outs[label] = engine.generate(prompts, max_new_tokens=10)
+        if label == "toy":
+            assert not model.capturable and engine.runner._graphs is None
+            assert "capturable" in engine.runner.graphs_refused
+            assert engine.warmup() == 0
+        elif label == "plain":
+            assert model.capturable and engine.runner._graphs
+        assert all(len(o) == 10 for o in outs[label])
+        assert not cache.open_rows
+    assert outs["toy"] == outs["toy-eager"]
+    with pytest.raises(KeyError, match="capturable = False"):
+        NoHostView()["seq_qstart"]
+
+
 # ---- a toy feed-forward with routing and a toy position encoding, registered from outside ------
 @dataclass(frozen=True)
 class RoutedSpec:
@@ -309,6 +349,8 @@ class RoutedSpec:
 
 
 class RoutedFeedForward:
+    capturable = False          # looks at the router's choice on the host (a device wait)
+
     @staticmethod
     def tensors(spec):
         t = {"router.weight": TensorDecl((spec.n_experts, spec.hidden), "vector")}
