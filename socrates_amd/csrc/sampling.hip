@@ -7,6 +7,10 @@
 // made, so a request's tokens do not depend on its neighbours in the batch. Every sum is
 // float32 and taken in a fixed order.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
+#include <stdio.h>
 
 constexpr int SAMPLE_THREADS = 1024;
 
@@ -144,6 +148,80 @@ SOC_EXPORT int soc_argmax(const float* logits, void* partial, int* out, int n, i
     hipLaunchKernelGGL(argmax_pick_kernel, dim3(n), dim3(SOC_WAVE), 0, stream, (const MaxIdx*)partial, out,
                        n_chunks);
     return soc_last_error();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Greedy choice without a workspace argument and without an allocation (see sampling.h): the
+// chunk results go to a file-scope device array. Host code never uses the array's name as an
+// address: it is looked up once per device with hipGetSymbolAddress, and the kernels get the
+// looked-up pointer as an argument, exactly as they get the caller's workspace in soc_argmax.
+static __device__ __align__(256) MaxIdx scratch[SOC_ARGMAX_STATIC_MAX_ROWS * SOC_ARGMAX_STATIC_MAX_CHUNKS];
+
+constexpr int STATIC_MAX_DEVICES = 64;
+static MaxIdx* scratch_of_device[STATIC_MAX_DEVICES];          // null until looked up
+static std::mutex scratch_lock;
+
+static void say(char* message, int message_len, const char* text, long a = 0, long b = 0) {
+    if (message && message_len > 0) snprintf(message, (size_t)message_len, text, a, b);
+}
+
+// The array's address on the current device, looked up at the first call on that device.
+static int static_scratch(MaxIdx** ptr, char* message, int message_len) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) {
+        say(message, message_len, "soc_argmax_static: hipGetDevice failed (HIP error %ld)", (long)err);
+        return (int)err;
+    }
+    if (device < 0 || device >= STATIC_MAX_DEVICES) {
+        say(message, message_len, "soc_argmax_static: device %ld is beyond the %ld this library keeps a pointer for",
+            device, STATIC_MAX_DEVICES);
+        return (int)hipErrorInvalidDevice;
+    }
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_of_device[device]) {
+        void* p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p) {
+            say(message, message_len, "soc_argmax_static: hipGetSymbolAddress failed on device %ld (HIP error %ld)",
+                device, (long)err);
+            return err != hipSuccess ? (int)err : (int)hipErrorInvalidSymbol;
+        }
+        scratch_of_device[device] = (MaxIdx*)p;
+    }
+    *ptr = scratch_of_device[device];
+    return 0;
+}
+
+SOC_EXPORT int soc_argmax_static_init(char* message, int message_len) {
+    MaxIdx* p = nullptr;
+    return static_scratch(&p, message, message_len);
+}
+
+SOC_EXPORT int soc_argmax_static(const float* logits, int* out, int n, int V, hipStream_t stream,
+                                 char* message, int message_len) {
+    if (n <= 0) return 0;
+    if (n > SOC_ARGMAX_STATIC_MAX_ROWS) {
+        say(message, message_len, "soc_argmax_static: %ld rows asked for, the static workspace holds %ld; "
+            "use soc_argmax with a workspace of your own", n, SOC_ARGMAX_STATIC_MAX_ROWS);
+        return (int)hipErrorInvalidValue;
+    }
+    if (V < 1 || !logits || !out) {
+        say(message, message_len, "soc_argmax_static: needs logits, out and a vocabulary of at least 1 (got %ld)", V);
+        return (int)hipErrorInvalidValue;
+    }
+    MaxIdx* partial = nullptr;
+    const int err = static_scratch(&partial, message, message_len);
+    if (err) return err;
+    const int n_chunks = max(1, min(SOC_ARGMAX_STATIC_MAX_CHUNKS, V / 2048));
+    const int chunk = (V + n_chunks - 1) / n_chunks;
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(n_chunks, n), dim3(ARGMAX_THREADS), 0, stream, logits,
+                       partial, V, chunk);
+    hipLaunchKernelGGL(argmax_pick_kernel, dim3(n), dim3(SOC_WAVE), 0, stream, (const MaxIdx*)partial, out,
+                       n_chunks);
+    const int launched = soc_last_error();
+    if (launched) say(message, message_len, "soc_argmax_static: launch failed (HIP error %ld)", launched);
+    return launched;
 }
 
 // logits [n, V] float32; temperature [n] float32 or null (all greedy); seed, draws [n] int64.

@@ -95,7 +95,8 @@ def _variant(name: str, head_dim=None):
 def _digest(name: str, defines) -> str:
     h = hashlib.sha256()
     h.update((CSRC / SOURCES[name]).read_bytes())
-    h.update((CSRC / "common.h").read_bytes())
+    for header in sorted(CSRC.glob("*.h")):
+        h.update(header.read_bytes())
     h.update(" ".join(HIPCC_FLAGS + list(defines)).encode())
     return h.hexdigest()[:12]
 
