@@ -119,6 +119,8 @@ def main(argv=None):
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-tune", action="store_true", help="library products with the library's default choice")
+    ap.add_argument("--no-fused-norms", action="store_true",
+                    help="decode steps with the residual sums and norms in kernels of their own")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is "
@@ -137,6 +139,7 @@ def main(argv=None):
     biggest = max(args.batch, 1 if args.no_points else 64)
     config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
     V = config.vocab_size
+    engine.runner.ops.fuse_norms = not args.no_fused_norms
     if args.dtype == "bf16" and not args.no_tune:
         # the library's products (more than 16 rows): its fastest solution for the prompt's shapes
         # and, up to 16 rows, the faster of the library and this package's own kernel for the timed batch

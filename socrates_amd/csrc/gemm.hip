@@ -216,12 +216,106 @@ template <int MT, int RW> struct SkBuf { uint4 w[RW][SK_UNROLL]; uint4 x[MT][SK_
 // gate tile and the second half the up tile, each half splitting K; the epilogue writes
 // silu(gate) * up, [M, N / 2], instead of both products. (One tile per wave streams the
 // weights faster than two.)
-template <typename TC, int MT, int RW, bool SWIGLU = false>
-__global__ void __launch_bounds__(64 * (SWIGLU ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES))
+//
+// Two more forms (one tile of 16 rows of x, one weight tile per workgroup, no split of K over
+// workgroups) take the residual sum and the RMSNorm out of a kernel of their own, for steps
+// of at most 16 tokens, where such a kernel costs as much as a small product:
+//  ADDNORM  the product is a branch's last projection. The epilogue adds it to the float32
+//           residual stream in place (a workgroup owns its 16 columns of every row), stores
+//           x' = bf16(h * gain) for the norm that follows, h being the new residual, and
+//           the sum of h^2 over its 16 columns per row: ssq [M, tiles rounded up to 4].
+//  SCALED   x is such an x' with its ssq. The norm's factor 1 / sqrt(mean(h^2) + eps) is the
+//           same for a whole row, so it is applied to the sums after the product instead of
+//           to x before it: out = (W x') / sqrt(sum_t ssq[m, t] / dim + eps). Statistics and
+//           factor stay float32; x' is rounded once, as the norm's output would be.
+struct SkNorm {
+    const float* ssq_in;        // SCALED: [M, ssq_tiles rounded up to a multiple of 4]
+    int ssq_tiles;
+    float inv_dim, eps;
+    float* residual;            // ADDNORM: [M, N] float32, updated in place
+    const float* gain;          // ADDNORM: [N], the following norm's weight
+    bf16* x_out;                // ADDNORM: [M, N]
+    float* ssq_out;             // ADDNORM: [M, gridDim.x rounded up to a multiple of 4]
+};
+constexpr int SK_SWIGLU = 1, SK_SCALED = 2, SK_ADDNORM = 4;
+constexpr int SK_SSQ_MAX_PAIRS = 16 * 16;       // 16 rows x 16 segments of 256 tiles: norms over up to 65,536 elements
+
+// SCALED: the factor of each of the 16 rows, from the partial sums of squares ssq [M, stride]
+// (stride: the tiles rounded up to a multiple of 4, so that rows start on 16 bytes). A wave
+// takes (row, segment of 256 tiles) pairs wave, wave + n_waves, ...; a lane loads four
+// consecutive tiles of its pair, so a row of up to 256 tiles is one load of one wave. The
+// first SK_SSQ_AHEAD pairs of a wave are asked for before the weights (no branch: a pair
+// outside the matrix loads the first element in all lanes, which costs one request, and is
+// left out of the sum), so that their way from memory is not waited for at the end.
+constexpr int SK_SSQ_AHEAD = 4;
+
+__device__ __forceinline__ int sk_ssq_stride(int tiles) { return (tiles + 3) & ~3; }
+
+__device__ __forceinline__ float4 sk_ssq_load(const SkNorm& nm, int M, int pair, int lane) {
+    const int row = pair % 16, t = (pair / 16) * 256 + lane * 4;
+    const float* p = (row < M && t < nm.ssq_tiles) ? nm.ssq_in + (size_t)row * sk_ssq_stride(nm.ssq_tiles) + t
+                                                   : nm.ssq_in;
+    return *reinterpret_cast<const float4*>(p);
+}
+
+__device__ __forceinline__ float sk_ssq_masked(const SkNorm& nm, int M, int pair, int lane, float4 v) {
+    const int row = pair % 16, t = (pair / 16) * 256 + lane * 4, T = nm.ssq_tiles;
+    float s = 0.f;
+    if (row < M) {                                     // in this order for every shape
+        s += t < T ? v.x : 0.f;
+        s += t + 1 < T ? v.y : 0.f;
+        s += t + 2 < T ? v.z : 0.f;
+        s += t + 3 < T ? v.w : 0.f;
+    }
+    return s;
+}
+
+__device__ __forceinline__ void sk_ssq_ahead(const SkNorm& nm, int M, int wave, int lane, float4 (&v)[SK_SSQ_AHEAD]) {
+    const int n_waves = blockDim.x / SOC_WAVE;
+#pragma unroll
+    for (int u = 0; u < SK_SSQ_AHEAD; ++u) v[u] = sk_ssq_load(nm, M, wave + u * n_waves, lane);
+}
+
+// Before the workgroup's barrier: the sum of each of this wave's pairs into LDS, part[pair].
+__device__ __forceinline__ void sk_ssq_shares(const SkNorm& nm, int M, int wave, int lane,
+                                              const float4 (&v)[SK_SSQ_AHEAD], float* part) {
+    const int n_waves = blockDim.x / SOC_WAVE;
+    const int pairs = 16 * ((nm.ssq_tiles + 255) / 256);
+#pragma unroll
+    for (int u = 0; u < SK_SSQ_AHEAD; ++u) {
+        const int pair = wave + u * n_waves;
+        const float s = wave_sum(sk_ssq_masked(nm, M, pair, lane, v[u]));
+        if (lane == 0 && pair < pairs && pair < SK_SSQ_MAX_PAIRS) part[pair] = s;
+    }
+    for (int pair = wave + SK_SSQ_AHEAD * n_waves; pair < pairs && pair < SK_SSQ_MAX_PAIRS; pair += n_waves) {
+        const float s = wave_sum(sk_ssq_masked(nm, M, pair, lane, sk_ssq_load(nm, M, pair, lane)));
+        if (lane == 0) part[pair] = s;
+    }
+}
+
+// After the barrier: the factor of row m, the same bits in every thread that asks.
+__device__ __forceinline__ float sk_row_factor(const SkNorm& nm, const float* part, int m) {
+    float total = 0.f;
+    for (int seg = 0; seg * 256 < nm.ssq_tiles; ++seg) total += part[seg * 16 + m];
+    return 1.0f / sqrtf(total * nm.inv_dim + nm.eps);
+}
+
+// waves of a workgroup: the forms with one tile of each operand may take 16 (their sums in
+// LDS stay small)
+__host__ __device__ constexpr int sk_max_waves(int MT, int RW, int MODE) {
+    return (MT * RW == 1 && (MODE & (SK_SWIGLU | SK_ADDNORM))) ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES;
+}
+
+template <typename TC, int MT, int RW, int MODE = 0>
+__global__ void __launch_bounds__(64 * sk_max_waves(MT, RW, MODE))
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
-                        int k_per_wave) {
-    __shared__ float red[(SWIGLU ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES) * MT * RW * 256];
+                        int k_per_wave, SkNorm nm) {
+    constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED, ADDNORM = MODE & SK_ADDNORM;
+    static_assert(!(SCALED || ADDNORM) || (MT == 1 && RW == 1), "the norm forms take one tile of each");
+    __shared__ float red[sk_max_waves(MT, RW, MODE) * MT * RW * 256];
+    __shared__ float norm_part[SCALED ? SK_SSQ_MAX_PAIRS : 1];      // [segment][16] sums of squares of the rows of x
+    __shared__ float sq_part[ADDNORM ? 16 * 16 : 1];        // [16][16] squares of the new residual
     // the wave index is the same in all lanes: say so, and the K loop runs on scalar registers
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
@@ -254,6 +348,17 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int r = 0; r < RW; ++r) acc[t][r] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // ADDNORM: the element of the residual and the gain that this thread's output meets, asked
+    // for ahead of the weights (every thread loads, from a clamped place: no branch here)
+    float4 ssq_v[SK_SSQ_AHEAD];
+    if constexpr (SCALED) sk_ssq_ahead(nm, M, wave, lane, ssq_v);
+    float old_h = 0.f, out_gain = 0.f;
+    if constexpr (ADDNORM) {
+        const int ln = (tid % 256) / 4, e = tid % 4;
+        const int m = min(ln % 16, M - 1), n = min(n0 + 4 * (ln / 16) + e, N - 1);
+        old_h = nm.residual[(size_t)m * N + n];
+        out_gain = nm.gain[n];
+    }
 
     // Full steps of 128 k load without any predicate (a weight row outside the matrix reads
     // row 0 and its results are dropped at the store; X rows outside read zeros through the
@@ -324,6 +429,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 red[(((wave * MT + t) * RW + r) * 64 + lane) * 4 + e] = acc[t][r][e];
+    if constexpr (SCALED) sk_ssq_shares(nm, M, wave, lane, ssq_v, norm_part);
     __syncthreads();
     if constexpr (SWIGLU) {
         static_assert(!SWIGLU || (RW == 1 && MT == 1), "one tile per wave, gate waves then up waves");
@@ -335,7 +441,34 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
                 u += red[((k_waves + w) * 64 + ln) * 4 + e];
             }
             const int m = ln % 16, col = blockIdx.x * 16 + 4 * (ln / 16) + e;
+            if constexpr (SCALED) { const float f = sk_row_factor(nm, norm_part, m); g *= f; u *= f; }
             if (m < M && 2 * col < N) C[(size_t)m * (N / 2) + col] = from_float<TC>(u * (g / (1.0f + expf(-g))));
+        }
+        return;
+    }
+    if constexpr (ADDNORM) {
+        // 256 outputs, one per thread of the first four waves: thread 4 * ln + e has row
+        // ln % 16 and column 4 * (ln / 16) + e of the tile
+        const int ln = (tid % 256) / 4, e = tid % 4;
+        const int m = ln % 16, c = 4 * (ln / 16) + e, n = n0 + c;
+        if (tid < 256) {
+            float sum = 0.f;
+            for (int w = 0; w < n_waves; ++w) sum += red[(w * 64 + ln) * 4 + e];
+            if constexpr (SCALED) sum *= sk_row_factor(nm, norm_part, m);
+            float h = 0.f;
+            if (m < M && n < N) {
+                h = old_h + sum;
+                nm.residual[(size_t)m * N + n] = h;
+                nm.x_out[(size_t)m * N + n] = from_float<bf16>(h * out_gain);
+            }
+            sq_part[m * 16 + c] = h * h;
+        }
+        __syncthreads();
+        if (tid < M) {
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ss += sq_part[tid * 16 + i];
+            nm.ssq_out[(size_t)tid * sk_ssq_stride(gridDim.x) + blockIdx.x] = ss;
         }
         return;
     }
@@ -345,6 +478,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
         float sum = 0.f;
         for (int w = 0; w < n_waves; ++w) sum += red[((w * MT * RW + tr) * 64 + ln) * 4 + e];
         const int m = t * 16 + ln % 16, n = n0 + r * 16 + 4 * (ln / 16) + e;
+        if constexpr (SCALED) sum *= sk_row_factor(nm, norm_part, m % 16);
         if (m < M && n < N) {
             if (Cpart) Cpart[((size_t)blockIdx.y * M + m) * N + n] = sum;
             else C[(size_t)m * N + n] = from_float<TC>(sum);
@@ -360,28 +494,72 @@ static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, in
     const int k_per_wave = ((k_per_split + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT, RW>), dim3((N + 16 * RW - 1) / (16 * RW), k_splits),
                        dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (TC*)C, Cpart, M, N,
-                       K, k_per_split, k_per_wave);
+                       K, k_per_split, k_per_wave, SkNorm{});
     return soc_last_error();
 }
 
 // x [M <= 16, K] times w [N, K]^T with gate and up rows interleaved in blocks of 16, then
 // silu(gate) * up: C [M, N / 2]. N a multiple of 32, K a multiple of 8.
+// ssq_in (may be null): x is a following norm's input x' = bf16(h * gain) with the partial
+// sums of squares ssq_in [M, ssq_tiles] of its rows h of `norm_dim` elements; the norm's
+// factor is applied to the sums (the SCALED form above). bfloat16 output only then.
 SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C, int M, int N, int K,
-                                           int c_dtype, int n_waves, hipStream_t stream) {
+                                           int c_dtype, int n_waves, const float* ssq_in, int ssq_tiles,
+                                           int norm_dim, float eps, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23) || N % 32) return (int)hipErrorInvalidValue;
     if (n_waves < 2 || n_waves > SK_MAX_WAVES_SWIGLU || n_waves % 2) return (int)hipErrorInvalidValue;
+    if (ssq_in && (ssq_tiles < 1 || ssq_tiles > 16 * SK_SSQ_MAX_PAIRS || norm_dim < 1 || c_dtype != 1))
+        return (int)hipErrorInvalidValue;
     const int k_waves = n_waves / 2;
     const int k_per_wave = ((K + k_waves - 1) / k_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
     const int k_per_split = k_per_wave * k_waves;
-    if (c_dtype == 0)
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 1, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+    SkNorm nm{};
+    nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
+    if (ssq_in)
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU | SK_SCALED>), dim3(N / 32, 1),
+                           dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (bf16*)C,
+                           (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm);
+    else if (c_dtype == 0)
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (float*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave);
+                           k_per_split, k_per_wave, nm);
     else
-        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, true>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
+        hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave);
+                           k_per_split, k_per_wave, nm);
+    return soc_last_error();
+}
+
+// The norm forms of the skinny product, M <= 16, one weight tile per workgroup, K not split
+// over workgroups. ssq_in (may be null): x is an x' with its partial sums of squares, as
+// above. residual (may be null): the product is added to residual [M, N] in place, and
+// x_out [M, N] = bf16(residual * gain), ssq_out [M, ceil(N / 16)] are written for the norm of
+// `N` elements that follows; C is then not written. At least one of the two is given.
+SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, int M, int N, int K,
+                                         int n_waves, const float* ssq_in, int ssq_tiles, int norm_dim,
+                                         float eps, float* residual, const float* gain, void* x_out,
+                                         float* ssq_out, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;
+    if (n_waves < 1 || n_waves > (residual ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES)) return (int)hipErrorInvalidValue;
+    if (!ssq_in && !residual) return (int)hipErrorInvalidValue;
+    if (ssq_in && (ssq_tiles < 1 || ssq_tiles > 16 * SK_SSQ_MAX_PAIRS || norm_dim < 1)) return (int)hipErrorInvalidValue;
+    if (residual ? (!gain || !x_out || !ssq_out) : !C) return (int)hipErrorInvalidValue;
+    if (residual) n_waves = max(n_waves, 4);            // its epilogue has one output per thread of four waves
+    const int k_per_wave = ((K + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
+    const int k_per_split = k_per_wave * n_waves;
+    SkNorm nm{};
+    nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
+    nm.residual = residual; nm.gain = gain; nm.x_out = (bf16*)x_out; nm.ssq_out = ssq_out;
+    const dim3 grid((N + 15) / 16, 1), block(n_waves * 64);
+#define SOC_SKN(MODE_) \
+    hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, MODE_>), grid, block, 0, stream, (const bf16*)X, \
+                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm)
+    if (ssq_in && residual) SOC_SKN(SK_SCALED | SK_ADDNORM);
+    else if (residual) SOC_SKN(SK_ADDNORM);
+    else SOC_SKN(SK_SCALED);
+#undef SOC_SKN
     return soc_last_error();
 }
 

@@ -17,8 +17,8 @@ import torch
 
 from .build import KernelBuildError, build_all, compile_library, load_library
 
-__all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "build_all", "compile_library",
-           "load_library", "plan_key_splits"]
+__all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "NormOwed", "build_all",
+           "compile_library", "load_library", "plan_key_splits"]
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -51,7 +51,8 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_mfma": [P, P, P, I, I, I, I, P],
     "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
-    "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P],
+    "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P, I, I, F, P],
+    "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -84,6 +85,22 @@ def plan_key_splits(n_blocks, n_kv_heads, group, max_keys):
     return split_len, (max_keys + split_len - 1) // split_len
 
 
+class NormOwed:
+    """Rows that are still owed their RMSNorm factor: ``x`` [M, dim] = bfloat16(h * gain) of the
+    rows h of the residual stream, and ``ssq`` [M, tiles rounded up to 4], float32 partial sums
+    of h^2 over tiles of 16 columns (the padding is never read). The factor 1 / sqrt(sum(ssq) / dim + eps) is one number per row, so the
+    product that consumes the rows applies it to its sums (``HipKernels.linear`` and
+    ``linear_swiglu`` take a NormOwed where they take x). Made by ``linear_add_norm``."""
+    __slots__ = ("x", "ssq", "dim", "eps")
+
+    def __init__(self, x, ssq, dim, eps):
+        self.x, self.ssq, self.dim, self.eps = x, ssq, dim, eps
+
+    @property
+    def shape(self):
+        return self.x.shape
+
+
 class HipKernels:
     def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
         if dtype not in _DTYPE_CODE:
@@ -114,6 +131,10 @@ class HipKernels:
         # package's tiled MFMA kernel
         self.library_gemm = True
         self.swiglu_waves = 8           # waves of the fused gate+up product (measured: 4, 8, 16 within 5 %)
+        # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
+        # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
+        self.fuse_norms = True
+        self.addnorm_waves = 0          # waves of such a projection, override
 
     # -- helpers -----------------------------------------------------------------------------
     def _stream(self):
@@ -204,6 +225,9 @@ class HipKernels:
     def linear_swiglu(self, x, w_gate_up, interleave=0):
         """swiglu(x @ w_gate_up^T). With rows interleaved in blocks of 16 and at most 16 rows of
         x in bfloat16, one kernel: the skinny product applies silu(gate) * up in its epilogue."""
+        owed = x if isinstance(x, NormOwed) else None
+        if owed is not None:
+            x = owed.x
         M, K = x.shape
         N = w_gate_up.shape[0]
         if (interleave == 16 and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
@@ -214,11 +238,51 @@ class HipKernels:
             n_waves = self.swiglu_waves          # half of them per tile (gate, up), splitting K
             while n_waves > 2 and K // (n_waves // 2) < 128:
                 n_waves //= 2
+            ssq, tiles, dim, eps = self._owed_args(owed, M, K)
             _check(self._gemm.soc_gemm_bf16_skinny_swiglu(_ptr(x), _ptr(w_gate_up), _ptr(out), c_int(M), c_int(N),
                                                           c_int(K), c_int(self.code), c_int(n_waves),
+                                                          ssq, c_int(tiles), c_int(dim), c_float(eps),
                                                           self._stream()), "linear_swiglu")
             return out
-        return self.swiglu(self.linear(x, w_gate_up), interleave)
+        return self.swiglu(self.linear(owed if owed is not None else x, w_gate_up), interleave)
+
+    def _owed_args(self, owed, M, K):
+        """(ssq pointer, tiles, dim, eps) of a NormOwed input, checked; nulls for a plain one."""
+        if owed is None:
+            return None, 0, 0, 0.0
+        if owed.dim != K:
+            raise KernelError(f"rows owed a norm over {owed.dim} elements meet a product over {K}")
+        tiles = (owed.dim + 15) // 16
+        self._want(owed.ssq, "sums of squares", torch.float32, (M, (tiles + 3) // 4 * 4))
+        return _ptr(owed.ssq), tiles, owed.dim, owed.eps
+
+    def linear_add_norm(self, y, w, residual, gain, eps):
+        """residual += y @ w^T, then the RMSNorm (``gain``, ``eps``) of the new residual: what
+        ``add_rmsnorm(residual, linear(y, w), gain, eps)`` returns. For bfloat16 steps of at most
+        16 rows it is one kernel: the product's epilogue adds to the residual and leaves the
+        rows as a NormOwed, whose factor the next product applies (``y`` may be one itself)."""
+        owed = y if isinstance(y, NormOwed) else None
+        yx = owed.x if owed is not None else y
+        (M, K), N = yx.shape, w.shape[0]
+        if not (self.dtype == torch.bfloat16 and yx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and self.fuse_norms):
+            return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps)
+        self._want(yx, "y")
+        self._want(w, "weight", None, (N, K))
+        self._want(residual, "residual", torch.float32, (M, N))
+        self._want(gain, "norm weight", torch.float32, (N,))
+        tiles = (N + 15) // 16
+        x_out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+        ssq_out = torch.empty((M, (tiles + 3) // 4 * 4), dtype=torch.float32, device=self.device)
+        n_waves = self.addnorm_waves or 8
+        while n_waves > 1 and K // n_waves < 128:
+            n_waves //= 2
+        ssq, in_tiles, dim, in_eps = self._owed_args(owed, M, K)
+        _check(self._gemm.soc_gemm_bf16_skinny_norm(
+            _ptr(yx), _ptr(w), None, c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(in_tiles),
+            c_int(dim), c_float(in_eps), _ptr(residual), _ptr(gain), _ptr(x_out), _ptr(ssq_out),
+            self._stream()), f"linear_add_norm [{M}x{K}] x [{N}x{K}]^T")
+        return NormOwed(x_out, ssq_out, N, eps)
 
     # -- matrix products ------------------------------------------------------------------------
     def library_tuning(self, on: bool) -> None:
@@ -268,6 +332,8 @@ class HipKernels:
         or this package's tiled MFMA kernel if ``library_gemm`` is off. ``allow_partial``: the consumer
         (the residual-add + norm kernel) accepts float32 split-K partial sums [S, M, N]; the
         skinny kernel then spreads a narrow output over more workgroups."""
+        if isinstance(x, NormOwed):
+            return self._linear_owed(x, w, out_dtype or self.dtype, n_waves)
         self._want(x, "x")
         self._want(w, "weight")
         if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -327,6 +393,29 @@ class HipKernels:
             err = self._gemm.soc_gemm_generic(*args, c_int(_DTYPE_CODE[x.dtype]), c_int(_DTYPE_CODE[w.dtype]),
                                               c_int(_DTYPE_CODE[out_dtype]), self._stream())
         _check(err, f"linear [{M}x{K}] x [{N}x{K}]^T")
+        return out
+
+    def _linear_owed(self, owed, w, out_dtype, n_waves=0):
+        """x' [M <= 16, K] of a NormOwed times w [N, K] transposed, the norm's factor applied
+        to the sums: one skinny product, bfloat16 out."""
+        x = owed.x
+        self._want(x, "x", torch.bfloat16)
+        self._want(w, "weight", torch.bfloat16)
+        if w.dim() != 2 or x.shape[1] != w.shape[1]:
+            raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(w.shape)}")
+        (M, K), N = x.shape, w.shape[0]
+        if out_dtype != torch.bfloat16 or not 0 < M <= 16 or K % 8:
+            raise KernelError("rows owed a norm go to bfloat16 products of at most 16 rows")
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+        if not n_waves:
+            n_waves = 8
+            while n_waves > 1 and K // n_waves < 128:
+                n_waves //= 2
+        ssq, tiles, dim, eps = self._owed_args(owed, M, K)
+        _check(self._gemm.soc_gemm_bf16_skinny_norm(
+            _ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(tiles),
+            c_int(dim), c_float(eps), None, None, None, None, self._stream()),
+            f"linear (norm owed) [{M}x{K}] x [{N}x{K}]^T")
         return out
 
     # -- attention pieces ----------------------------------------------------------------------

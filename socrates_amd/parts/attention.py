@@ -50,7 +50,10 @@ class PagedAttention:
                          if spec.position is not None else None)
         self.capturable = getattr(self.position, "capturable", True)
 
-    def forward(self, x, ctx, slot, write=True):
+    takes_projection = True     # the block may supply the last product
+    takes_norm_owed = True      # x goes to one product only
+
+    def forward(self, x, ctx, slot, write=True, project=None):
         s, ops = self.spec, self.ops
         Hq, Hkv, D = s.n_heads, s.n_kv_heads, s.head_dim
         if write:
@@ -72,6 +75,8 @@ class PagedAttention:
             if write:
                 ops.kv_write(k, v, ctx.positions, ctx.token_rows, slot)
         o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
+        if project is not None:
+            return project(o, self.w_o)
         # the block's next norm adds this output to the residual: partial sums are welcome
         return ops.linear(o, self.w_o, allow_partial=True)
 

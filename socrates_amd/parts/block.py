@@ -43,9 +43,21 @@ def _sub_tensors(spec: BlockSpec, role: str, weights):
     return {local: weights[prefix + local] for local in tensors_of(sub)}
 
 
+class Normed:
+    """What a branch returns when its last projection has already added its output to the
+    residual stream and computed the following norm: ``rows`` is that norm's output (a
+    tensor, or whatever the kernel set hands the next product in its place)."""
+    __slots__ = ("rows",)
+
+    def __init__(self, rows):
+        self.rows = rows
+
+
 class PreNormBlock:
+    chains = True       # forward takes ``nxt``, the block that runs after this one
+
     def __init__(self, spec: BlockSpec, weights, ops):
-        self.spec = spec
+        self.spec, self.ops = spec, ops
         self.norm1 = build_part(spec.norm1, _sub_tensors(spec, "norm1", weights), ops)
         self.mixer = build_part(spec.mixer, _sub_tensors(spec, "mixer", weights), ops)
         self.norm2 = build_part(spec.norm2, _sub_tensors(spec, "norm2", weights), ops)
@@ -55,13 +67,28 @@ class PreNormBlock:
         self.capturable = all(getattr(p, "capturable", True)
                               for p in (self.norm1, self.mixer, self.norm2, self.ffn))
 
-    def forward(self, residual, pending, ctx, slot, write=True):
+    def _branch(self, part, args, residual, norm, consumer):
+        """Run a mixer or feed-forward. If the part ends with a projection that it lets the
+        block supply (``takes_projection``), the norm after it can be left to the kernel set
+        (``fusable``) and the part after that norm takes what the kernel set then returns in
+        place of normed rows (``takes_norm_owed``), the part's last product adds to the
+        residual stream and prepares the norm itself: one kernel instead of two."""
+        ops = self.ops
+        if (getattr(part, "takes_projection", False) and norm is not None and hasattr(norm, "fusable")
+                and getattr(consumer, "takes_norm_owed", False) and hasattr(ops, "linear_add_norm")):
+            gain, eps = norm.fusable()
+            return part.forward(*args, project=lambda y, w: Normed(ops.linear_add_norm(y, w, residual, gain, eps)))
+        return part.forward(*args)
+
+    def forward(self, residual, pending, ctx, slot, write=True, nxt=None):
         """residual: fp32 [N, hidden], updated in place. pending: the previous block's
-        un-added output or None. Returns this block's un-added feed-forward output."""
-        h = self.norm1.add_norm(residual, pending)
-        a = self.mixer.forward(h, ctx, slot, write)
-        h = self.norm2.add_norm(residual, a)
-        return self.ffn.forward(h, ctx)
+        un-added output, None, or a ``Normed`` (already added, and normed by this block's
+        first norm). ``nxt``: the block that runs next, if it is of this arrangement.
+        Returns this block's feed-forward output, un-added or as a ``Normed``."""
+        h = pending.rows if isinstance(pending, Normed) else self.norm1.add_norm(residual, pending)
+        a = self._branch(self.mixer, (h, ctx, slot, write), residual, self.norm2, self.ffn)
+        h = a.rows if isinstance(a, Normed) else self.norm2.add_norm(residual, a)
+        return self._branch(self.ffn, (h, ctx), residual, getattr(nxt, "norm1", None), getattr(nxt, "mixer", None))
 
 
 register_arrangement("prenorm", PreNormBlock)

@@ -31,8 +31,13 @@ class SwiGLU:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
-    def forward(self, x, ctx=None):
+    takes_projection = True     # the block may supply the last product
+    takes_norm_owed = True      # x goes to one product only
+
+    def forward(self, x, ctx=None, project=None):
         act = self.ops.linear_swiglu(x, self.w_gate_up, self.interleave)
+        if project is not None:
+            return project(act, self.w_down)
         # the block's next norm adds this output to the residual: partial sums are welcome
         return self.ops.linear(act, self.w_down, allow_partial=True)
 

@@ -62,9 +62,16 @@ class DecoderModel:
         ops = self.ops
         residual = ops.embedding(ctx.token_ids, self.embed)
         pending = None
-        for step in self.plan.order:
-            pending = self.blocks[step.layer].forward(
-                residual, pending, ctx, cache.slot(step.cache), step.write)
+        order = self.plan.order
+        for i, step in enumerate(order):
+            block = self.blocks[step.layer]
+            if getattr(block, "chains", False):
+                # the block may leave its last sum and the next block's first norm to its last product
+                nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
+                pending = block.forward(residual, pending, ctx, cache.slot(step.cache), step.write,
+                                        nxt=nxt if getattr(nxt, "chains", False) else None)
+            else:
+                pending = block.forward(residual, pending, ctx, cache.slot(step.cache), step.write)
         if ctx.n_want == 0:
             # The cache is complete after the last block; no logits are asked for.
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=ops.device)

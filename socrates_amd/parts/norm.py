@@ -27,6 +27,11 @@ class RMSNorm:
         """
         return self.ops.add_rmsnorm(residual, delta, self.weight, self.spec.eps, rows)
 
+    def fusable(self):
+        """(gain, eps): all a kernel set needs to compute this norm inside the products
+        around it (``HipKernels.linear_add_norm``)."""
+        return self.weight, self.spec.eps
+
     def __call__(self, x):
         """Plain norm over the last dimension of ``x`` (any leading shape)."""
         return self.ops.rmsnorm(x, self.weight, self.spec.eps)

@@ -149,6 +149,58 @@ def test_linear_split_k_partials(kernel_sets, M, N, K):
     hip.library_gemm = True
 
 
+@pytest.mark.parametrize("M,d,K,eps", [(1, 64, 64, 1e-6), (8, 2560, 4096, 1e-6), (16, 72, 200, 1e-5),
+                                       (5, 100, 9728, 1e-2), (3, 4096, 96, 1e-6), (11, 2560, 9728, 1e-6)])
+def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
+    """A projection that adds to the residual stream and leaves the norm's factor to the
+    next product (one kernel), against product, sum and norm one after the other: the new
+    residual, then the three kinds of product that can consume the rows. Rows are scaled very
+    differently, so a factor applied to the wrong row, or left out, shows."""
+    from socrates_amd.kernels import NormOwed
+    hip, ref = kernel_sets[torch.bfloat16]
+    y, w = rnd((M, K), torch.bfloat16, 40), rnd((d, K), torch.bfloat16, 41, K ** -0.5)
+    res = rnd((M, d), torch.float32, 42) * torch.logspace(-2, 2, M, device=DEV)[:, None]
+    gain = (1 + 0.3 * torch.randn(d)).to(DEV)
+    want_res = res.double() + y.double() @ w.double().T
+    want_normed = (want_res * torch.rsqrt((want_res ** 2).mean(-1, keepdim=True) + eps) * gain.double())
+    r = res.clone()
+    owed = hip.linear_add_norm(y, w, r, gain, eps)
+    tiles = (d + 15) // 16
+    assert isinstance(owed, NormOwed) and owed.ssq.shape == (M, (tiles + 3) // 4 * 4)
+    torch.testing.assert_close(r.double(), want_res, atol=2e-2, rtol=1e-2)
+    torch.testing.assert_close(owed.ssq[:, :tiles].double().sum(-1), (r.double() ** 2).sum(-1), atol=1e-6, rtol=1e-5)
+    owed.ssq[:, tiles:] = float("nan")           # the padding is never read
+    # the exact values the kernel should have stored, from its own residual
+    torch.testing.assert_close(owed.x, (r * gain).to(torch.bfloat16), atol=0, rtol=0)
+    normed = (r.double() * torch.rsqrt((r.double() ** 2).mean(-1, keepdim=True) + eps) * gain.double())
+    torch.testing.assert_close(normed, want_normed, atol=2e-2, rtol=2e-2)
+    # consumers: a plain product, gate / up with the activation, and another projection with a sum
+    if d % 8 == 0:
+        N2 = 331 if d < 1000 else 6144
+        w2 = rnd((N2, d), torch.bfloat16, 43, d ** -0.5)
+        close(hip.linear(owed, w2), normed @ w2.double().T, torch.bfloat16)
+        ff = 160 if d < 1000 else 9728
+        gate, up = rnd((ff, d), torch.bfloat16, 44, d ** -0.5), rnd((ff, d), torch.bfloat16, 45, d ** -0.5)
+        wgu = torch.stack([gate.view(ff // 16, 16, d), up.view(ff // 16, 16, d)], 1).reshape(2 * ff, d).contiguous()
+        want = torch.nn.functional.silu(normed @ gate.double().T) * (normed @ up.double().T)
+        close(hip.linear_swiglu(owed, wgu, 16), want, torch.bfloat16)
+        w3 = rnd((88, d), torch.bfloat16, 46, d ** -0.5)
+        res3 = rnd((M, 88), torch.float32, 47)
+        gain3 = (1 + 0.3 * torch.randn(88)).to(DEV)
+        r3 = res3.clone()
+        owed3 = hip.linear_add_norm(owed, w3, r3, gain3, 1e-5)
+        torch.testing.assert_close(r3.double(), res3.double() + normed @ w3.double().T, atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(owed3.x, (r3 * gain3).to(torch.bfloat16), atol=0, rtol=0)
+    # more than 16 rows, or the switch off: the same call is product, then sum and norm
+    hip.fuse_norms = False
+    r = res.clone()
+    plain = hip.linear_add_norm(y, w, r, gain, eps)
+    hip.fuse_norms = True
+    assert isinstance(plain, torch.Tensor)
+    close(plain, want_normed, torch.bfloat16, atol=3e-2)
+    torch.testing.assert_close(r.double(), want_res, atol=2e-2, rtol=1e-2)
+
+
 def test_linear_float32_is_not_reduced_precision(kernel_sets):
     """Values that bfloat16 or a 19-bit matrix mode would round away survive."""
     hip, _ = kernel_sets[torch.float32]
