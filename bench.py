@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine at Qwen3-4B size on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--preset qwen3-8b]
+    python bench.py --mixed [--preset qwen3-8b] [--requests 160]
 
 A step is one decode step of the engine: plan, run the batch through the model from
 the cache, sample, read the tokens back. Random weights (seeded), prompts of uniform
@@ -22,7 +23,8 @@ sys.path.insert(0, str(ROOT))
 HBM_GBPS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-DEFAULT_PRESET = "qwen3-4b"        # socrates_amd/config/presets/qwen3-4b.json: BASELINE.json configs[2]
+DEFAULT_PRESET = "qwen3-4b"        # socrates_amd/config/presets/qwen3-4b.json, the headline configuration
+MIXED_PRESET = "qwen3-8b"          # the serving workload's: prompt portions beside decoding rows
 
 
 def preset_dict(name):
@@ -32,17 +34,17 @@ def preset_dict(name):
     return json.loads(preset_path(name).read_text())
 
 
-def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_):
+def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_, chunk=2048):
     import torch
 
     from socrates_amd.cache import CacheManager, blocks_for
-    from socrates_amd.config import Qwen3Config
+    from socrates_amd.config import config_class_for
     from socrates_amd.engine import Engine, ModelRunner
     from socrates_amd.kernels import HipKernels
     from socrates_amd.parts import DecoderModel, cache_needs, expected_tensors
     from socrates_amd.weights import random_tensors
 
-    config = Qwen3Config.from_dict(cfg_dict)
+    config = config_class_for(cfg_dict["architectures"][0]).from_dict(cfg_dict)
     plan = config.plan()
     ops = HipKernels(dtype, "cuda:0")
     weights = random_tensors(expected_tensors(plan), seed, dtype=dtype, device="cuda:0")
@@ -52,8 +54,83 @@ def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_):
                          num_blocks=max_batch * blocks_for(max_len, 16), dtype=dtype, device="cuda:0")
     runner = ModelRunner(model, cache)
     engine = Engine(runner, max_batch=max_batch, max_len=max_len, max_new_tokens=max_len,
-                    chunk=2048, compile=compile_)
+                    chunk=chunk, compile=compile_)
     return config, engine
+
+
+def mixed_workload(args, dtype):
+    """The serving workload: requests with prompts of uniform length in [128, 4096] arrive all
+    at once; up to ``--decode-rows`` of them decode while the next prompt is run in portions
+    of up to 2,048 tokens beside them (the step's token budget is the portion plus the rows).
+    Every step is timed on the host around the engine's whole step (plan, run, sample, read
+    back) and sorted by what it ran. Prints one JSON line; ``value`` is all tokens (prompt
+    and generated) per second over the whole run."""
+    import torch
+
+    from socrates_amd.sampling import SamplingParams
+    cfg = preset_dict(args.preset)
+    full_layers = cfg["num_hidden_layers"]
+    layers = args.layers or full_layers
+    cfg["num_hidden_layers"] = layers
+    rows, portion = args.decode_rows, args.prefill_tokens
+    config, engine = build_engine(cfg, dtype, rows + 1, args.max_len, seed=0, compile_=not args.no_graphs,
+                                  chunk=portion + rows)
+    engine.runner.ops.fuse_norms = not args.no_fused_norms
+    if args.dtype == "bf16" and not args.no_tune:
+        engine.tune([portion + rows, rows])
+    rng = random.Random(7)
+    params = SamplingParams(max_new_tokens=args.new_tokens, eos_token_ids=())
+    reqs = [engine.submit([rng.randrange(config.vocab_size) for _ in range(rng.randint(128, 4096))], sampling=params)
+            for _ in range(args.requests)]
+    kinds = {"mixed": [0, 0.0, 0, 0], "prompt_only": [0, 0.0, 0, 0], "decode_only": [0, 0.0, 0, 0]}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while not engine.scheduler.idle:
+        a = time.perf_counter()
+        n = engine.step()
+        b = time.perf_counter()
+        if n == 0:
+            if engine.scheduler.idle:           # the last requests were retired by this call
+                break
+            raise RuntimeError("requests are waiting but nothing can be scheduled")
+        lens = engine.last_portions
+        n_decode = sum(1 for t in lens if t == 1)
+        kind = "decode_only" if n_decode == len(lens) else ("mixed" if n_decode else "prompt_only")
+        k = kinds[kind]
+        k[0] += 1
+        k[1] += b - a
+        k[2] += n
+        k[3] += n_decode
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    new = sum(len(r.output) for r in reqs)
+    prompt = sum(len(r.ids) for r in reqs)
+    sized = {"qwen3-4b": "Qwen3-4B-sized", "qwen3-8b": "Qwen3-8B-sized", "qwen3-32b": "Qwen3-32B-sized"}.get(
+        args.preset, args.preset)
+    summary = {kind: {"steps": k[0], "ms_per_step": round(k[1] / k[0] * 1e3, 3), "tokens_per_step": round(k[2] / k[0], 1),
+                      "decode_rows_per_step": round(k[3] / k[0], 1), "tok_s": round(k[2] / k[1], 1)}
+               for kind, k in kinds.items() if k[0]}
+    out = {
+        "metric": f"tokens/s through mixed steps: portions of up to {portion} prompt tokens beside up to {rows} "
+                  f"decoding rows ({sized}, {args.dtype})",
+        "value": round((prompt + new) / dt, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": sum(k[0] for k in kinds.values()), "warmup": 0,
+        "ms_per_step": round(dt / sum(k[0] for k in kinds.values()) * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: seeded random weights, uniform random token ids, prompt lengths uniform in [128, 4096]",
+        "config": {"model": sized, "global_batch": rows, "seq_len": args.max_len, "parallelism": "single GPU",
+                   "layers": layers, "layers_full": full_layers, "hidden_size": config.hidden_size,
+                   "num_attention_heads": config.num_attention_heads,
+                   "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+                   "intermediate_size": config.intermediate_size, "vocab_size": config.vocab_size,
+                   "requests": args.requests, "new_tokens_per_request": args.new_tokens,
+                   "portion_tokens": portion, "block_size": 16, "hip_graphs": not args.no_graphs},
+        "new_tok_s": round(new / dt, 1), "prompt_tokens": prompt, "new_tokens": new, "seconds": round(dt, 3),
+        "preemptions": engine.scheduler.n_preemptions,
+    }
+    out.update(summary)
+    print(json.dumps(out))
+    return 0
 
 
 def decode_rate(engine, batch, context, steps, warmup, vocab, seed):
@@ -112,7 +189,13 @@ def main(argv=None):
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--max-len", type=int, default=4096)
-    ap.add_argument("--preset", default=DEFAULT_PRESET, help="a configuration of socrates_amd/config/presets")
+    ap.add_argument("--preset", default=None, help="a configuration of socrates_amd/config/presets "
+                    f"(default {DEFAULT_PRESET}; with --mixed {MIXED_PRESET})")
+    ap.add_argument("--mixed", action="store_true",
+                    help="the serving workload: prompt portions beside decoding rows (see mixed_workload)")
+    ap.add_argument("--requests", type=int, default=160, help="--mixed: requests in the run")
+    ap.add_argument("--new-tokens", type=int, default=128, help="--mixed: tokens generated per request")
+    ap.add_argument("--decode-rows", type=int, default=64, help="--mixed: requests that decode side by side")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--no-graphs", action="store_true")
@@ -130,6 +213,11 @@ def main(argv=None):
     import torch
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     item = 2 if args.dtype == "bf16" else 4
+    if args.mixed:
+        args.preset = args.preset or MIXED_PRESET
+        args.max_len = max(args.max_len, 8192)
+        return mixed_workload(args, dtype)
+    args.preset = args.preset or DEFAULT_PRESET
     cfg = preset_dict(args.preset)
     full_layers = cfg["num_hidden_layers"]
     args.layers = args.layers or full_layers

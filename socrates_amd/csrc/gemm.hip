@@ -236,6 +236,8 @@ struct SkNorm {
     const float* gain;          // ADDNORM: [N], the following norm's weight
     bf16* x_out;                // ADDNORM: [M, N]
     float* ssq_out;             // ADDNORM: [M, gridDim.x rounded up to a multiple of 4]
+    float* split_sums;          // ADDNORM with K split over workgroups: [tiles, splits, 256], scratch
+    int* split_count;           // the same: [tiles], zero before the launch and after it
 };
 constexpr int SK_SWIGLU = 1, SK_SCALED = 2, SK_ADDNORM = 4;
 constexpr int SK_SSQ_MAX_PAIRS = 16 * 16;       // 16 rows x 16 segments of 256 tiles: norms over up to 65,536 elements
@@ -303,7 +305,7 @@ __device__ __forceinline__ float sk_row_factor(const SkNorm& nm, const float* pa
 // waves of a workgroup: the forms with one tile of each operand may take 16 (their sums in
 // LDS stay small)
 __host__ __device__ constexpr int sk_max_waves(int MT, int RW, int MODE) {
-    return (MT * RW == 1 && (MODE & (SK_SWIGLU | SK_ADDNORM))) ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES;
+    return MT * RW == 1 ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES;
 }
 
 template <typename TC, int MT, int RW, int MODE = 0>
@@ -316,6 +318,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     __shared__ float red[sk_max_waves(MT, RW, MODE) * MT * RW * 256];
     __shared__ float norm_part[SCALED ? SK_SSQ_MAX_PAIRS : 1];      // [segment][16] sums of squares of the rows of x
     __shared__ float sq_part[ADDNORM ? 16 * 16 : 1];        // [16][16] squares of the new residual
+    __shared__ bool split_last;
     // the wave index is the same in all lanes: say so, and the K loop runs on scalar registers
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
@@ -451,10 +454,39 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
         // ln % 16 and column 4 * (ln / 16) + e of the tile
         const int ln = (tid % 256) / 4, e = tid % 4;
         const int m = ln % 16, c = 4 * (ln / 16) + e, n = n0 + c;
+        float sum = 0.f;
         if (tid < 256) {
-            float sum = 0.f;
             for (int w = 0; w < n_waves; ++w) sum += red[(w * 64 + ln) * 4 + e];
             if constexpr (SCALED) sum *= sk_row_factor(nm, norm_part, m);
+        }
+        if (gridDim.y > 1) {
+            // K is split over gridDim.y workgroups per tile. Each leaves its 256 sums in memory
+            // and is counted; the one counted last adds all of them, in the order of the
+            // splits whoever came last, and goes on alone. No fence (a fence writes back and
+            // invalidates this chip's whole L2, which costs more than the kernel): the sums
+            // are written through the caches and read past them (agent-scope atomic stores and
+            // loads), and a wait for the stores' acknowledgement orders them before the count.
+            float* mine = nm.split_sums + ((size_t)blockIdx.x * gridDim.y + blockIdx.y) * 256;
+            if (tid < 256) __hip_atomic_store(mine + tid, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) {
+                const int before = __hip_atomic_fetch_add(nm.split_count + blockIdx.x, 1, __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT);
+                split_last = before == (int)gridDim.y - 1;
+                // the count is left at zero for the next launch that uses it
+                if (split_last) __hip_atomic_store(nm.split_count + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            if (!split_last) return;
+            if (tid < 256) {
+                const float* all = nm.split_sums + (size_t)blockIdx.x * gridDim.y * 256 + tid;
+                sum = 0.f;
+                for (int sp = 0; sp < (int)gridDim.y; ++sp)
+                    sum += __hip_atomic_load(all + sp * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (tid < 256) {
             float h = 0.f;
             if (m < M && n < N) {
                 h = old_h + sum;
@@ -536,23 +568,31 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
 // above. residual (may be null): the product is added to residual [M, N] in place, and
 // x_out [M, N] = bf16(residual * gain), ssq_out [M, ceil(N / 16)] are written for the norm of
 // `N` elements that follows; C is then not written. At least one of the two is given.
+// k_splits > 1 (with residual only): K is split over that many workgroups per tile, which meet
+// through split_sums [ceil(N / 16), k_splits, 256] floats (scratch) and split_count
+// [ceil(N / 16)] ints, which must be zero before the call and are zero again after it. Two
+// launches that may run at the same time need counts of their own.
 SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, int M, int N, int K,
                                          int n_waves, const float* ssq_in, int ssq_tiles, int norm_dim,
                                          float eps, float* residual, const float* gain, void* x_out,
-                                         float* ssq_out, hipStream_t stream) {
+                                         float* ssq_out, int k_splits, float* split_sums, int* split_count,
+                                         hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;
-    if (n_waves < 1 || n_waves > (residual ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES)) return (int)hipErrorInvalidValue;
+    if (n_waves < 1 || n_waves > SK_MAX_WAVES_SWIGLU) return (int)hipErrorInvalidValue;
     if (!ssq_in && !residual) return (int)hipErrorInvalidValue;
     if (ssq_in && (ssq_tiles < 1 || ssq_tiles > 16 * SK_SSQ_MAX_PAIRS || norm_dim < 1)) return (int)hipErrorInvalidValue;
     if (residual ? (!gain || !x_out || !ssq_out) : !C) return (int)hipErrorInvalidValue;
     if (residual) n_waves = max(n_waves, 4);            // its epilogue has one output per thread of four waves
-    const int k_per_wave = ((K + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
+    if (k_splits < 1 || k_splits > 64 || (k_splits > 1 && (!residual || !split_sums || !split_count)))
+        return (int)hipErrorInvalidValue;
+    const int k_per_wave = ((K + k_splits * n_waves - 1) / (k_splits * n_waves) + SK_STEP - 1) / SK_STEP * SK_STEP;
     const int k_per_split = k_per_wave * n_waves;
     SkNorm nm{};
+    nm.split_sums = split_sums; nm.split_count = split_count;
     nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
     nm.residual = residual; nm.gain = gain; nm.x_out = (bf16*)x_out; nm.ssq_out = ssq_out;
-    const dim3 grid((N + 15) / 16, 1), block(n_waves * 64);
+    const dim3 grid((N + 15) / 16, k_splits), block(n_waves * 64);
 #define SOC_SKN(MODE_) \
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, MODE_>), grid, block, 0, stream, (const bf16*)X, \
                        (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm)
@@ -591,7 +631,8 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
                                     hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;   // 32-bit byte offsets into X
-    if (n_waves < 1 || n_waves > SK_MAX_WAVES || k_splits < 1 || k_splits > 65535)
+    if (n_waves < 1 || n_waves > (M <= 16 && row_tiles == 1 ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES) || k_splits < 1 ||
+        k_splits > 65535)
         return (int)hipErrorInvalidValue;
     if ((k_splits > 1) != (Cpart != nullptr)) return (int)hipErrorInvalidValue;
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);

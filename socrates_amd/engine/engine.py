@@ -63,6 +63,7 @@ class Engine:
         if compile and hasattr(self.runner, "enable_graphs"):
             self.runner.enable_graphs(max_batch)
         self.n_steps = 0
+        self.last_portions: List[int] = []      # tokens of each request in the last step (1: a decoded token)
         self.prompt_tokens = 0          # counters in place of the reference's Prometheus ones
         self.output_tokens = 0
 
@@ -115,6 +116,7 @@ class Engine:
             return 0
         entries = [StepEntry(p.request.row, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
                    for p in plan]
+        self.last_portions = [len(p.tokens) for p in plan]
         logits = self.runner.step(entries, borrow=True)
         wanted = [p for p in plan if p.wants_logits]
         tokens = self.sampler.sample(logits, [p.request.row for p in wanted])

@@ -52,7 +52,7 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, P],
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
     "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P, I, I, F, P],
-    "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, P],
+    "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, I, P, P, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -135,6 +135,11 @@ class HipKernels:
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
         self.fuse_norms = True
         self.addnorm_waves = 0          # waves of such a projection, override
+        self.addnorm_splits = 0         # workgroups that share one tile's K in it, override
+        # arrival counts of those workgroups, one per tile of 16 outputs: zero between launches
+        # (the last to arrive leaves it so). All launches of this kernel set share them, so
+        # they must not overlap: one stream, as everywhere in this package.
+        self._split_count = torch.zeros(16384, dtype=torch.int32, device=self.device)
 
     # -- helpers -----------------------------------------------------------------------------
     def _stream(self):
@@ -278,11 +283,35 @@ class HipKernels:
         while n_waves > 1 and K // n_waves < 128:
             n_waves //= 2
         ssq, in_tiles, dim, in_eps = self._owed_args(owed, M, K)
+        k_splits = self.addnorm_splits or self._addnorm_splits(tiles, K)
+        while k_splits > 1 and K // (k_splits * n_waves) < 128:
+            k_splits //= 2
+        sums = count = None
+        if k_splits > 1:
+            if tiles > self._split_count.numel():
+                raise KernelError(f"linear_add_norm: {N} outputs are more than the {16 * self._split_count.numel()} "
+                                  "that K can be split for")
+            sums = torch.empty((tiles, k_splits, 256), dtype=torch.float32, device=self.device)
+            count = self._split_count
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(yx), _ptr(w), None, c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(in_tiles),
             c_int(dim), c_float(in_eps), _ptr(residual), _ptr(gain), _ptr(x_out), _ptr(ssq_out),
-            self._stream()), f"linear_add_norm [{M}x{K}] x [{N}x{K}]^T")
+            c_int(k_splits), _ptr(sums), _ptr(count), self._stream()), f"linear_add_norm [{M}x{K}] x [{N}x{K}]^T")
         return NormOwed(x_out, ssq_out, N, eps)
+
+    @staticmethod
+    def _addnorm_splits(tiles, K):
+        """Workgroups that share one tile's K in ``linear_add_norm``. Measured on an MI355X at
+        the output and down projections of 4B-, 8B- and 32B-sized layers (tiles 160, 256, 320;
+        K 4,096 to 25,600; 1, 8 and 16 rows): meeting in memory costs about 2 us, so K is split
+        only where a tile per workgroup leaves the GPU unevenly filled (the tiles are no
+        multiple of its 256 compute units) and every wave keeps some 300 elements of K."""
+        if tiles % 256 == 0:
+            return 1
+        splits = 4
+        while splits > 1 and K // (splits * 8) < 300:
+            splits //= 2
+        return splits
 
     # -- matrix products ------------------------------------------------------------------------
     def library_tuning(self, on: bool) -> None:
@@ -414,7 +443,7 @@ class HipKernels:
         ssq, tiles, dim, eps = self._owed_args(owed, M, K)
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(tiles),
-            c_int(dim), c_float(eps), None, None, None, None, self._stream()),
+            c_int(dim), c_float(eps), None, None, None, None, c_int(1), None, None, self._stream()),
             f"linear (norm owed) [{M}x{K}] x [{N}x{K}]^T")
         return out
 

@@ -163,6 +163,22 @@ def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
     gain = (1 + 0.3 * torch.randn(d)).to(DEV)
     want_res = res.double() + y.double() @ w.double().T
     want_normed = (want_res * torch.rsqrt((want_res ** 2).mean(-1, keepdim=True) + eps) * gain.double())
+    # K split over 2 or 4 workgroups per tile that meet in memory (twice each: the arrival
+    # counts must be back at zero after a call); the sums must not depend on who comes last
+    hip.addnorm_splits = 1
+    r = res.clone()
+    first = hip.linear_add_norm(y, w, r, gain, eps)
+    for splits in (2, 4, 4, 2):
+        hip.addnorm_splits = splits
+        r_s = res.clone()
+        owed_s = hip.linear_add_norm(y, w, r_s, gain, eps)
+        torch.testing.assert_close(r_s, r, atol=2e-3, rtol=1e-4)
+        torch.testing.assert_close(owed_s.x, (r_s * gain).to(torch.bfloat16), atol=0, rtol=0)
+        again = res.clone()
+        hip.linear_add_norm(y, w, again, gain, eps)
+        assert torch.equal(again, r_s)
+    hip.addnorm_splits = 0
+    assert int(hip._split_count.abs().sum()) == 0
     r = res.clone()
     owed = hip.linear_add_norm(y, w, r, gain, eps)
     tiles = (d + 15) // 16
