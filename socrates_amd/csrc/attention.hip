@@ -343,20 +343,31 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        int table_width, const int* __restrict__ token_rows,
                        const int* __restrict__ positions, const int* __restrict__ row_blocks,
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
-                       float* __restrict__ part_ml, int Hq, int Hkv, int BS, int bs_shift, float scale,
-                       int window, int split_len, int n_splits, int group_pad_log2) {
-    __shared__ __attribute__((aligned(16))) uint16_t v_lds[4][16 * V_STRIDE];
+                       float* __restrict__ part_ml, int* __restrict__ arrivals, int Hq, int Hkv, int BS,
+                       int bs_shift, float scale, int window, int split_len, int n_splits,
+                       int group_pad_log2) {
+    // One piece of LDS: the waves' V tiles while the keys are walked; afterwards, with key
+    // splits, what the four waves of the workgroup have gathered, to be combined.
+    constexpr int V_BYTES = 4 * 16 * V_STRIDE * 2, C_BYTES = 4 * RT * DV * 64 * 16;
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[V_BYTES > C_BYTES ? V_BYTES : C_BYTES];
+    __shared__ float c_ml[4][RT][16][2];
+    __shared__ int came_last;
+    uint16_t (*v_lds)[16 * V_STRIDE] = reinterpret_cast<uint16_t (*)[16 * V_STRIDE]>(lds_raw);
     // the wave index is the same in all lanes: say so, and what depends on it (the task, its
     // token, position and table row) is computed and loaded on the scalar side
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / SOC_WAVE), lane = threadIdx.x % SOC_WAVE;
     const int G = Hq / Hkv;
     const int Gp = 1 << group_pad_log2;                 // rows per token in a row block
     const int chunks = (G + 15) / 16;                   // head chunks when G > 16
-    const int task = blockIdx.x * 4 + wave;
+    // Without key splits the four waves of a workgroup take four tasks. With splits
+    // (a multiple of four) they take four consecutive splits of one task, combine what they
+    // find through LDS, and the workgroups of a task (n_splits / 4 of them) meet in memory.
+    const bool by_split = n_splits > 1;
+    const int task = by_split ? (int)blockIdx.x : (int)blockIdx.x * 4 + wave;
     if (task >= n_row_blocks * Hkv * chunks) return;
     const int blk = task / (Hkv * chunks);
     const int kvh = (task / chunks) % Hkv, chunk = task % chunks;
-    const int split = blockIdx.y;
+    const int split = by_split ? (int)blockIdx.y * 4 + wave : 0;
     // no list of row blocks: every token alone (a decode step), one dependent load fewer
     const int tok0 = row_blocks ? row_blocks[2 * blk] : blk, ntok = row_blocks ? row_blocks[2 * blk + 1] : 1;
     const int pos0 = positions[tok0];
@@ -590,141 +601,157 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     }
 
     // finish: the row sum is spread over the four lanes of the row's column
+    float L[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        float L = l[rt];
-        L = sum_xor32(sum_xor16(L));
-        if (row_pos[rt] < 0) continue;
-        const size_t base = row_q[rt];                                   // (token * Hq + head) * D
-        if (n_splits == 1) {
-            const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int rt = 0; rt < RT; ++rt) L[rt] = sum_xor32(sum_xor16(l[rt]));
+    if (!by_split) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            if (row_pos[rt] < 0) continue;
+            const float inv = L[rt] > 0.f ? 1.0f / L[rt] : 0.f;
 #pragma unroll
             for (int j = 0; j < DV; ++j) {
                 uint2 pk;
-                pk.x = (uint32_t)f32_to_bf16_bits(o[rt][j][0] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][1] * inv) << 16);
-                pk.y = (uint32_t)f32_to_bf16_bits(o[rt][j][2] * inv) | ((uint32_t)f32_to_bf16_bits(o[rt][j][3] * inv) << 16);
-                *reinterpret_cast<uint2*>(out + base + j * 16 + 4 * kb) = pk;
+                pk.x = pack_bf16x2(o[rt][j][0] * inv, o[rt][j][1] * inv);
+                pk.y = pack_bf16x2(o[rt][j][2] * inv, o[rt][j][3] * inv);
+                *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
             }
-        } else {
-            // partials lie by (row block, token in it), not by token: a call may cover some of
-            // the tokens only
-            const long shift = row_blocks ? (long)blk * ((16 * RT) >> group_pad_log2) - tok0 : 0;
-            const size_t pi = (size_t)((long)(base / D) + shift * Hq) * n_splits + split;
-            if (m[rt] != -INFINITY) {                        // the merge reads nothing of an empty split
+        }
+        return;
+    }
+    // Four splits, one per wave, through LDS: every wave leaves its sums and its references,
+    // then takes every fourth 16-wide block of the head dimension and adds the four shares of
+    // it under a common reference (any reference serves, see the lazy maximum above).
+    float4 (*c_o)[RT * DV][64] = reinterpret_cast<float4 (*)[RT * DV][64]>(lds_raw);
+    __syncthreads();                                        // every wave is done with its V tiles
 #pragma unroll
-                for (int j = 0; j < DV; ++j)
-                    *reinterpret_cast<float4*>(part_o + pi * D + j * 16 + 4 * kb) =
-                        make_float4(o[rt][j][0], o[rt][j][1], o[rt][j][2], o[rt][j][3]);
+    for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int j = 0; j < DV; ++j)
+            c_o[wave][rt * DV + j][lane] = make_float4(o[rt][j][0], o[rt][j][1], o[rt][j][2], o[rt][j][3]);
+        if (kb == 0) { c_ml[wave][rt][li][0] = m[rt]; c_ml[wave][rt][li][1] = L[rt]; }
+    }
+    __syncthreads();
+    const int outer = n_splits / 4;                         // workgroups of this task
+    // partials lie by (row block, token in it), not by token: a call may cover some of the
+    // tokens only
+    const long shift = row_blocks ? (long)blk * ((16 * RT) >> group_pad_log2) - tok0 : 0;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        float wgt[4], M4 = -INFINITY, L4 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M4 = fmaxf(M4, c_ml[w][rt][li][0]);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = c_ml[w][rt][li][0];
+            wgt[w] = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M4);
+            L4 += wgt[w] * c_ml[w][rt][li][1];
+        }
+        if (row_pos[rt] < 0) continue;
+        const size_t pi = (size_t)((long)(row_q[rt] / D) + shift * Hq) * outer + blockIdx.y;
+        const float inv = L4 > 0.f ? 1.0f / L4 : 0.f;
+        for (int j = wave; j < DV; j += 4) {
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float4 t = c_o[w][rt * DV + j][lane];
+                a.x += t.x * wgt[w]; a.y += t.y * wgt[w]; a.z += t.z * wgt[w]; a.w += t.w * wgt[w];
             }
-            if (kb == 0) { part_ml[pi * 2] = m[rt]; part_ml[pi * 2 + 1] = L; }
+            if (outer == 1) {
+                uint2 pk;
+                pk.x = pack_bf16x2(a.x * inv, a.y * inv);
+                pk.y = pack_bf16x2(a.z * inv, a.w * inv);
+                *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
+            } else {
+                // written through the caches (agent scope): another workgroup reads it below
+                float* dst = part_o + pi * D + j * 16 + 4 * kb;
+                __hip_atomic_store(dst, a.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + 1, a.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + 2, a.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + 3, a.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (outer > 1 && wave == 0 && kb == 0) {
+            __hip_atomic_store(part_ml + pi * 2, M4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(part_ml + pi * 2 + 1, L4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-}
-
-// Merge all n_splits partials of a (token, head); an empty split has m = -inf and is not
-// read. One wave per (token, head): first the splits lie across the lanes (maximum, weights,
-// sum); then a lane owns four elements of the head dimension and every D / 4 lanes form a
-// group that adds every (64 / (D / 4))-th split, in order; the groups are added in order.
-__global__ void __launch_bounds__(64)
-paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                        bf16* __restrict__ out, int Hq, int n_splits,
-                        const int* __restrict__ row_blocks, int tokens_per_block) {
-    constexpr int LPG = D / 4;                              // lanes of a group
-    constexpr int NG = SOC_WAVE / LPG;                      // groups of a wave
-    __shared__ float weight[256];
-    __shared__ __attribute__((aligned(16))) float4 red[SOC_WAVE];
-    const int h = blockIdx.x, lane = threadIdx.x;
-    int n = blockIdx.y;                                     // the token; its partials lie at blockIdx.y
-    if (row_blocks) {
-        const int blk = blockIdx.y / tokens_per_block, j = blockIdx.y % tokens_per_block;
-        if (j >= row_blocks[2 * blk + 1]) return;
-        n = row_blocks[2 * blk] + j;
+    if (outer == 1) return;
+    // The workgroups of a task meet in memory without a fence (a fence writes back and
+    // invalidates the chip's whole L2): the partial results above went through the caches, a
+    // wait for their acknowledgement orders them before the arrival count, and the workgroup
+    // counted last reads all of them past the caches and writes the rows. The count is left
+    // at zero for the next launch.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int before = __hip_atomic_fetch_add(arrivals + task, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        came_last = before == outer - 1;
+        if (came_last) __hip_atomic_store(arrivals + task, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    const size_t base = ((size_t)blockIdx.y * Hq + h) * n_splits;
-    constexpr int FAST = 32;                                // partials a lane holds on the short path
-    if (n_splits <= SOC_WAVE && n_splits <= FAST * NG) {
-        // Few splits: every load is issued before any is needed (one trip to memory instead
-        // of two). An empty split's partial was never written: it is loaded, but not used.
-        const int sg = lane / LPG, e4 = lane % LPG;
-        const float ms = lane < n_splits ? part_ml[(base + lane) * 2] : -INFINITY;
-        const float ls = lane < n_splits ? part_ml[(base + lane) * 2 + 1] : 0.f;
-        float4 v[FAST];
-#pragma unroll
-        for (int j = 0; j < FAST; ++j) {
-            const int s = sg + j * NG;
-            v[j] = (sg < NG && s < n_splits)
-                       ? *reinterpret_cast<const float4*>(part_o + (base + s) * D + e4 * 4)
-                       : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        const float M = wave_max(ms);
-        const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);   // the maxima are in base 2
-        const float L = wave_sum(w * ls);
-        const float inv = L > 0.f ? 1.0f / L : 0.f;
+    __syncthreads();
+    if (!came_last) return;
+    // The rows of the task go round the four waves. For a row, the splits' references and sums
+    // lie across the lanes (at most 64 workgroups per task); a lane owns four elements of the
+    // head dimension, every D / 4 lanes form a group, and group g adds the splits g, g + NG, ...
+    // in that order; the groups are added in order. All loads of a round are issued before the
+    // first is needed: one trip to memory for a row.
+    constexpr int LPG = D / 4, NG = SOC_WAVE / LPG, ROUND = 8;
+    float4* red = reinterpret_cast<float4*>(lds_raw) + wave * SOC_WAVE;
+    const int sg = lane / LPG, e4 = lane % LPG;
+    for (int rho = wave; rho < 16 * RT; rho += 4) {
+        const int tt = rho >> group_pad_log2, g = chunk * 16 + ((rho % 16) & (Gp - 1));
+        if (tt >= ntok || g >= G) continue;
+        const size_t row = (size_t)(tok0 + tt) * Hq + (size_t)kvh * G + g;       // (token, head)
+        const size_t p0 = (size_t)((long)row + shift * Hq) * outer;
+        const int mine = lane < outer ? lane : 0;
+        const float ms_ = __hip_atomic_load(part_ml + (p0 + mine) * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float ls_ = __hip_atomic_load(part_ml + (p0 + mine) * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        float M = 0.f, Lt = 0.f, wl = 0.f;
+        for (int s0 = 0; s0 < outer; s0 += ROUND * NG) {
+            float4 v[ROUND];
 #pragma unroll
-        for (int j = 0; j < FAST; ++j) {
-            const int s = sg + j * NG;
-            const float wj = __shfl(w, s < SOC_WAVE ? s : 0, SOC_WAVE);
-            if (sg < NG && s < n_splits && wj != 0.f) {
-                acc.x += v[j].x * wj; acc.y += v[j].y * wj; acc.z += v[j].z * wj; acc.w += v[j].w * wj;
+            for (int j = 0; j < ROUND; ++j) {
+                const int sp = s0 + sg + j * NG;
+                const float* src = part_o + (p0 + (sg < NG && sp < outer ? sp : 0)) * D + e4 * 4;
+                v[j].x = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[j].y = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[j].z = __hip_atomic_load(src + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[j].w = __hip_atomic_load(src + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (s0 == 0) {
+                const float ms = lane < outer ? ms_ : -INFINITY;
+                M = wave_max(ms);
+                wl = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);      // the references are in base 2
+                Lt = wave_sum(wl * (lane < outer ? ls_ : 0.f));
+            }
+#pragma unroll
+            for (int j = 0; j < ROUND; ++j) {
+                const int sp = s0 + sg + j * NG;
+                const float wj = __shfl(wl, sp < SOC_WAVE ? sp : 0, SOC_WAVE);
+                if (sg < NG && sp < outer && wj != 0.f) {
+                    acc.x += v[j].x * wj; acc.y += v[j].y * wj; acc.z += v[j].z * wj; acc.w += v[j].w * wj;
+                }
             }
         }
         if constexpr (NG > 1) {
             red[lane] = acc;
-            __syncthreads();
-            if (lane < LPG) {
-                for (int g = 1; g < NG; ++g) {
-                    const float4 t = red[g * LPG + lane];
+            __builtin_amdgcn_wave_barrier();
+            if (lane < LPG)
+                for (int gi = 1; gi < NG; ++gi) {
+                    const float4 t = red[gi * LPG + lane];
                     acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
                 }
-            }
+            __builtin_amdgcn_wave_barrier();
         }
         if (lane < LPG) {
+            const float inv = Lt > 0.f ? 1.0f / Lt : 0.f;
             uint2 pk;
             pk.x = pack_bf16x2(acc.x * inv, acc.y * inv);
             pk.y = pack_bf16x2(acc.z * inv, acc.w * inv);
-            *reinterpret_cast<uint2*>(out + ((size_t)n * Hq + h) * D + e4 * 4) = pk;
+            *reinterpret_cast<uint2*>(out + row * D + e4 * 4) = pk;
         }
-        return;
-    }
-    float M = -INFINITY;
-    for (int s = lane; s < n_splits; s += SOC_WAVE) M = fmaxf(M, part_ml[(base + s) * 2]);
-    M = wave_max(M);
-    float lsum = 0.f;                                       // the launcher allows at most 256 splits
-    for (int s = lane; s < n_splits; s += SOC_WAVE) {
-        const float ms = part_ml[(base + s) * 2];
-        const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - M);
-        weight[s] = w;
-        lsum += w * part_ml[(base + s) * 2 + 1];
-    }
-    const float L = wave_sum(lsum);
-    __syncthreads();
-    const float inv = L > 0.f ? 1.0f / L : 0.f;
-    const int sg = lane / LPG, e4 = lane % LPG;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (sg < NG) {
-        for (int s = sg; s < n_splits; s += NG) {
-            const float w = weight[s];
-            if (w == 0.f) continue;
-            const float4 v = *reinterpret_cast<const float4*>(part_o + (base + s) * D + e4 * 4);
-            acc.x += v.x * w; acc.y += v.y * w; acc.z += v.z * w; acc.w += v.w * w;
-        }
-    }
-    if constexpr (NG > 1) {
-        red[lane] = acc;
-        __syncthreads();
-        if (lane < LPG) {
-            for (int g = 1; g < NG; ++g) {
-                const float4 v = red[g * LPG + lane];
-                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-            }
-        }
-    }
-    if (lane < LPG) {
-        uint2 pk;
-        pk.x = pack_bf16x2(acc.x * inv, acc.y * inv);
-        pk.y = pack_bf16x2(acc.z * inv, acc.w * inv);
-        *reinterpret_cast<uint2*>(out + ((size_t)n * Hq + h) * D + e4 * 4) = pk;
     }
 }
 
@@ -732,32 +759,37 @@ paged_attn_merge_kernel(const float* __restrict__ part_o, const float* __restric
 // (16 * row_tiles) >> group_pad_log2 tokens of one sequence, or null: every token is a block
 // of its own (n_row_blocks = N); 2^group_pad_log2 >= min(G, 16).
 // Splits are over absolute key indices: split s covers keys [s * split_len, (s + 1) * split_len),
-// split_len a multiple of 16; n_splits > 1 needs part_o [R, Hq, n_splits, D] and part_ml
-// [R, Hq, n_splits, 2] with R = N without row blocks, else n_row_blocks * tokens per block
-// (the blocks may cover some of the N tokens only; the others' outputs are not touched);
-// part_ml is written for every (row, split), empty ones with m = -inf.
+// split_len a multiple of 16. n_splits > 1 must be a multiple of 4 (four splits share a
+// workgroup), at most 256, and needs part_o [R, Hq, n_splits / 4, D] and part_ml
+// [R, Hq, n_splits / 4, 2] if n_splits > 4, with R = N without row blocks, else n_row_blocks *
+// tokens per block (the blocks may cover some of the N tokens only; the others' outputs are
+// not touched), and `arrivals`, one int per task (row block x kv head x chunk of 16 heads),
+// zero before the call and zero again after it; calls that may run at the same time need
+// arrival counts of their own.
 SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const void* v_pool,
                                         const int* block_table, int table_width, const int* token_rows,
                                         const int* positions, const int* row_blocks, int n_row_blocks,
-                                        void* out, float* part_o, float* part_ml, int N, int Hq, int Hkv,
-                                        int BS, float scale, int window, int split_len, int n_splits,
-                                        int row_tiles, int group_pad_log2, hipStream_t stream) {
+                                        void* out, float* part_o, float* part_ml, int* arrivals, int N,
+                                        int Hq, int Hkv, int BS, float scale, int window, int split_len,
+                                        int n_splits, int row_tiles, int group_pad_log2, hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
         return (int)hipErrorInvalidValue;
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
-    if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
+    if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;
+    if (n_splits > 4 && (!part_o || !part_ml || !arrivals)) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
-    if (n_splits > 256) return (int)hipErrorInvalidValue;        // the merge holds 256 weights
+    if (n_splits > 256) return (int)hipErrorInvalidValue;
     if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
-    const dim3 grid((unsigned)((tasks + 3) / 4), n_splits);
+    if (tasks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    const dim3 grid = n_splits > 1 ? dim3((unsigned)tasks, n_splits / 4) : dim3((unsigned)((tasks + 3) / 4), 1);
     int bs_shift = -1;                                           // log2 of the page size if it is a power of two
     if ((BS & (BS - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
-        token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, Hq, Hkv, BS, bs_shift, \
+        token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
         scale, window, split_len, n_splits, group_pad_log2
     // Row tiles beyond what the registers hold at this head size are refused: two up to head
     // size 128, four up to 64.
@@ -780,13 +812,6 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     }
 #undef SOC_MFMA_LAUNCH
 #undef SOC_MFMA_ARGS
-    int err = soc_last_error();
-    if (err || n_splits == 1) return err;
-    const int tokens_per_block = (16 * row_tiles) >> group_pad_log2;
-    const long merge_rows = row_blocks ? (long)n_row_blocks * tokens_per_block : (long)N;
-    if (merge_rows > 65535) return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL(paged_attn_merge_kernel, dim3(Hq, (unsigned)merge_rows), dim3(64), 0, stream, part_o, part_ml,
-                       (bf16*)out, Hq, n_splits, row_blocks, tokens_per_block > 0 ? tokens_per_block : 1);
     return soc_last_error();
 }
 

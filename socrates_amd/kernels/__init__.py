@@ -57,7 +57,7 @@ _GEMM_SIGNATURES = {
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
-    "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
+    "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
     "soc_attention_head_dim": [],
 }
@@ -69,20 +69,24 @@ def _declare(lib, signatures):
         fn.argtypes, fn.restype = argtypes, (None if name.endswith("_plan") else c_int)
 
 
-MAX_KEY_SPLITS = 256    # what the merge kernel of the MFMA attention holds weights for
+MAX_KEY_SPLITS = 256    # of the MFMA attention: 64 workgroups of four splits meet per task
 
 
 def plan_key_splits(n_blocks, n_kv_heads, group, max_keys):
     """(split_len, n_splits) for the MFMA attention kernel: enough waves to fill the GPU, no
     split shorter than 64 keys, at most MAX_KEY_SPLITS of them (a longer context gets longer
-    splits). Splits are over absolute key indices, a multiple of 16 keys long, and cover keys
-    0 .. max_keys - 1. Host arithmetic only."""
+    splits), one split or a multiple of four (four share a workgroup; some of the last four
+    may lie beyond the keys and are empty). Splits are over absolute key indices, a multiple of
+    16 keys long, and cover keys 0 .. max_keys - 1. Host arithmetic only."""
     waves = n_blocks * n_kv_heads * ((group + 15) // 16)
-    # from one wave per SIMD on (1,024) no split: the merge costs a wave per (token, head)
+    # from one wave per SIMD on (1,024) no split: a split costs a trip through LDS, or memory
     n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64,
                                            MAX_KEY_SPLITS))
+    if n == 1:
+        return ((max_keys + 15) // 16 * 16), 1
+    n = (n + 3) // 4 * 4
     split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
-    return split_len, (max_keys + split_len - 1) // split_len
+    return split_len, ((max_keys + split_len - 1) // split_len + 3) // 4 * 4
 
 
 class NormOwed:
@@ -586,8 +590,10 @@ class HipKernels:
             split_len, n_splits = self.attention_splits
             split_len = max(16, (min(split_len, 1 << 24) + 15) // 16 * 16)
             n_splits = max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
+            if n_splits > 1:
+                n_splits = (n_splits + 3) // 4 * 4          # four splits share a workgroup
             if n_splits > MAX_KEY_SPLITS:
-                raise KernelError(f"{n_splits} key splits asked for; the MFMA attention kernel merges at "
+                raise KernelError(f"{n_splits} key splits asked for; the MFMA attention kernel takes at "
                                   f"most {MAX_KEY_SPLITS}")
             return split_len, n_splits
         return plan_key_splits(n_blocks, n_kv_heads, group, max_keys)
@@ -602,15 +608,20 @@ class HipKernels:
         blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block, which)
         split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
         part_o = part_ml = None
-        if n_splits > 1:
+        if n_splits > 4:
+            # the workgroups of a task (four splits each) meet in memory
+            tasks = n_blocks * Hkv * ((G + 15) // 16)
+            if tasks > self._split_count.numel():
+                raise KernelError(f"{tasks} (row block, kv head) pairs with key splits: more than the "
+                                  f"{self._split_count.numel()} arrival counts held")
             part_rows = N if blocks is None else n_blocks * tokens_per_block
-            part_o = torch.empty((part_rows, Hq, n_splits, D), dtype=torch.float32, device=self.device)
-            part_ml = torch.empty((part_rows, Hq, n_splits, 2), dtype=torch.float32, device=self.device)
+            part_o = torch.empty((part_rows, Hq, n_splits // 4, D), dtype=torch.float32, device=self.device)
+            part_ml = torch.empty((part_rows, Hq, n_splits // 4, 2), dtype=torch.float32, device=self.device)
         _check(lib.soc_paged_attention_mfma(
             _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
             c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
-            c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), c_int(N), c_int(Hq), c_int(Hkv),
-            c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
+            c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(self._split_count), c_int(N),
+            c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
             c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
 
     def paged_attention(self, q, slot, ctx, scale, window=None):

@@ -7,9 +7,10 @@ from socrates_amd.kernels import MAX_KEY_SPLITS, plan_key_splits
 
 @pytest.mark.parametrize("n_kv_heads", [1, 2, 4, 8])
 def test_key_splits_stay_within_what_the_merge_holds(n_kv_heads):
-    """Rows 1..64, groups 1..16, contexts up to 131,072 keys: never more splits than the merge
-    kernel holds weights for, splits are whole 16-key tiles, and together they cover every key
-    (the last split may be short, none is empty)."""
+    """Rows 1..64, groups 1..16, contexts up to 131,072 keys: never more splits than the
+    kernel takes, one split or a multiple of four (four share a workgroup), splits are whole
+    16-key tiles, and together they cover every key (the last may be short; of the last four
+    some may be empty, never all)."""
     keys = [1, 15, 16, 17, 255, 256, 257, 1000, 2048, 4096, 16448, 20000, 32768, 65536, 100000, 131072]
     for rows in list(range(1, 18)) + [24, 32, 48, 64]:
         for group in range(1, 17):
@@ -17,8 +18,9 @@ def test_key_splits_stay_within_what_the_merge_holds(n_kv_heads):
                 split_len, n = plan_key_splits(rows, n_kv_heads, group, max_keys)
                 assert 1 <= n <= MAX_KEY_SPLITS, (rows, group, max_keys, n)
                 assert split_len % 16 == 0 and split_len >= 16
+                assert n == 1 or n % 4 == 0
                 assert n * split_len >= max_keys                  # covers the keys
-                assert (n - 1) * split_len < max_keys             # and no split is empty
+                assert (n - (1 if n == 1 else 4)) * split_len < max_keys    # and no workgroup is empty
 
 
 def test_key_splits_cases_that_used_to_exceed_the_limit():
@@ -28,5 +30,5 @@ def test_key_splits_cases_that_used_to_exceed_the_limit():
     split_len, n = plan_key_splits(1, 2, 4, 20000)
     assert n <= 256 and n * split_len >= 20000
     # a short context is not cut below 64 keys, a full launch is not cut at all
-    assert plan_key_splits(1, 8, 4, 100)[1] <= 2
+    assert plan_key_splits(1, 8, 4, 100)[1] <= 4
     assert plan_key_splits(128, 8, 4, 4096) == (4096, 1)
