@@ -274,7 +274,8 @@ class HipKernels:
         yx = owed.x if owed is not None else y
         (M, K), N = yx.shape, w.shape[0]
         if not (self.dtype == torch.bfloat16 and yx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and self.fuse_norms):
+                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N <= 65536 and self.fuse_norms):
+            # (65,536: the sums of squares of a row are summed by one wave per 256 tiles of 16)
             return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps)
         self._want(yx, "y")
         self._want(w, "weight", None, (N, K))

@@ -106,11 +106,21 @@ def load_weights(folder, expected, compute_dtype, device):
     if missing or unexpected or wrong_shape or wrong_dtype:
         raise WeightError(folder, missing, unexpected, wrong_shape, wrong_dtype)
     out = {}
+    kept_wide = []
     for f, items in by_file.items():
         with safe_open(str(f), framework="pt") as sf:
             for name, decl in items:
                 stored = sf.get_slice(name).get_dtype()
                 t = sf.get_tensor(name)
-                out[name] = t.to(device=device, dtype=kept_dtype(decl.kind, stored, compute_dtype)
-                                 ).contiguous()
+                dtype = kept_dtype(decl.kind, stored, compute_dtype)
+                if decl.kind not in ("int", "vector") and dtype != compute_dtype:
+                    kept_wide.append(name)
+                out[name] = t.to(device=device, dtype=dtype).contiguous()
+    if kept_wide:
+        # a matrix stored in 32-bit stays 32-bit: said aloud, because its products then take
+        # the plain float32 kernel and the matrix twice the memory
+        import warnings
+        warnings.warn(f"{folder}: {len(kept_wide)} matrices are stored in 32-bit floats and are kept so under "
+                      f"{compute_dtype} (first: {kept_wide[0]}); their products run in the float32 kernel. "
+                      "Store the checkpoint in bfloat16 for the fast path.", stacklevel=2)
     return out

@@ -90,6 +90,24 @@ def test_bf16_cuts_agree_with_each_other(folders, oracle, name):
         torch.testing.assert_close(results["mixed"][rid], results["whole"][rid], atol=3e-2, rtol=3e-2)
 
 
+@pytest.mark.parametrize("name", list(TINIES))
+def test_short_steps_with_the_norms_in_kernels_of_their_own(folders, oracle, name):
+    """Steps of at most 16 tokens fold the residual sums and norms into the products around
+    them; with that switched off the same steps run product, sum and norm one after the other.
+    Both ways match the oracle, and agree with each other far more closely than with it; the
+    arrival counts that workgroups meet through are back at zero afterwards."""
+    prompts, want = oracle[name]
+    results = {}
+    for fused in (True, False):
+        runner = runner_for(folders[name], TINIES[name], torch.bfloat16, 64)
+        runner.ops.fuse_norms = fused
+        results[fused] = replay(runner, trace_tail_decode(prompts, 32))
+        compare(results[fused], want, torch.bfloat16, f"{name}/tail32/fused={fused}")
+        assert int(runner.ops._split_count.abs().sum()) == 0
+    for rid in results[True]:
+        torch.testing.assert_close(results[True][rid], results[False][rid], atol=3e-2, rtol=3e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_first_tokens_and_long_decode(folders, dtype):
     """The first tokens of a sequence one by one (positions 0, 1, 2 ...), then a long
