@@ -336,7 +336,29 @@ __device__ __forceinline__ void rescale_in_place(f32x4_t (&o)[RT_][DV_], const f
     scale_fence();
 }
 
-template <int RT, bool TP>
+// FUSED (decode steps: every token alone; one row tile; head sizes in steps of 32, and of 64
+// with a rotation, which is over the whole head): q is not given. The kernel reads the token's raw
+// [q heads | k heads | v heads] row as the QKV product left it, and does what
+// qk_norm_rope_kernel does on its way: per-head RMSNorm of q and k (if gains are given), the
+// rotation at the token's position, all in float32 with one rounding to bfloat16. A lane's
+// slices of a head hold both partners of every rotated pair, so nothing crosses lanes but the
+// sum of squares. The token's own key and value do not go through the cache: the wave whose
+// split holds the token's position adds them as one more tile from registers, and (for one
+// chunk of heads) stores them to the page for the steps to come. The work hides behind the
+// start of the walk (position -> table -> first keys), which it does not depend on.
+struct FusedQkv {
+    const bf16* qkv;            // [N, row_heads, D]: q heads, then (if the step writes the slot) k and v heads
+    int row_heads;
+    const float* q_gain;        // [D] each, or null: no norm
+    const float* k_gain;
+    const float* rope_table;    // [positions][2][D / 2] cosines and sines (soc_rope_table), or null: no rotation
+    float eps;
+    int write_kv;               // the step writes this cache slot (else it only reads it: queries only)
+    bf16* k_pool_w;             // the pools again, to write to
+    bf16* v_pool_w;
+};
+
+template <int RT, bool TP, bool FUSED = false>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                        const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -345,7 +367,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
                        float* __restrict__ part_ml, int* __restrict__ arrivals, int Hq, int Hkv, int BS,
                        int bs_shift, float scale, int window, int split_len, int n_splits,
-                       int group_pad_log2) {
+                       int group_pad_log2, FusedQkv fz) {
+    static_assert(!FUSED || (RT == 1 && QK_K32), "the fused form: one row tile, head sizes in steps of 32");
     // One piece of LDS: the waves' V tiles while the keys are walked; afterwards, with key
     // splits, what the four waves of the workgroup have gathered, to be combined.
     constexpr int V_BYTES = 4 * 16 * V_STRIDE * 2, C_BYTES = 4 * RT * DV * 64 * 16;
@@ -375,7 +398,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 
     // keys this wave walks: its split, cut to what its rows can see
     int klo = split * split_len;
-    int khi = min(klo + split_len, pos0 + ntok);
+    // FUSED and writing: the token's own key is not read from the cache (it is not there yet)
+    const bool own_key = FUSED && fz.write_kv;
+    const bool covers = pos0 >= klo && pos0 < klo + split_len;      // this wave's split holds the token's position
+    int khi = min(klo + split_len, own_key ? pos0 : pos0 + ntok);
     if (window > 0) klo = max(klo, pos0 - window + 1);
     const int kmin = klo;                                // first key any row of the block can see
     klo = klo & ~15;                                     // tiles are aligned to 16 keys
@@ -393,9 +419,106 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         const bool ok = tt < ntok && g < G;
         row_pos[rt] = ok ? pos0 + tt : -1;
         row_q[rt] = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? g : 0)) * D;
+        if constexpr (!FUSED) {
 #pragma unroll
-        for (int kk = 0; kk < QK_STEPS; ++kk)
-            qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
+            for (int kk = 0; kk < QK_STEPS; ++kk)
+                qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
+        }
+    }
+    __shared__ float rope_cs[FUSED ? 4 : 1][FUSED ? D : 1];          // cos [0, D / 2), sin [D / 2, D) of the wave's token
+    __shared__ uint4 new_kv[FUSED ? 4 : 1][FUSED ? 2 * (D / 8) : 1]; // the token's key (normed, rotated) and value, by 16-byte part
+    if constexpr (FUSED) {
+        const bf16* row_in = fz.qkv + (size_t)tok0 * fz.row_heads * D;
+        const int g = chunk * 16 + (li & (Gp - 1));
+        const bool ok = row_pos[0] >= 0;
+        // raw slices first: the row's query head, the kv head's key, one part of its value
+        // (every wave loads; without k and v heads in the row, a query head stands in and is
+        // not used)
+        const size_t q_at = ((size_t)kvh * G + (ok ? g : 0)) * D;
+        const size_t k_at = own_key ? (size_t)(Hq + kvh) * D : q_at, v_at = own_key ? (size_t)(Hq + Hkv + kvh) * D : q_at;
+        uint4 qraw[QK_STEPS], kraw[QK_STEPS];
+#pragma unroll
+        for (int kk = 0; kk < QK_STEPS; ++kk) {
+            qraw[kk] = load_qk_slice(row_in + q_at, kk, kb);
+            kraw[kk] = load_qk_slice(row_in + k_at, kk, kb);
+        }
+        const uint4 vraw = *reinterpret_cast<const uint4*>(row_in + v_at + (lane % (D / 8)) * 8);
+        // the token's cosines and sines, from the table (an accurate sincosf in each of a
+        // launch's thousands of waves would cost more vector time than the walk itself)
+        if (fz.rope_table) {
+            const float* cs_row = fz.rope_table + (size_t)pos0 * D;
+            for (int j = lane; j < D; j += SOC_WAVE) rope_cs[wave][j] = cs_row[j];
+            __builtin_amdgcn_wave_barrier();
+        }
+        // norm and rotation of this lane's slices of one head: elements 32 kk + 8 kb + t; the
+        // partner of an element of the first half lies QK_STEPS / 2 slices on, in the same lane
+        auto norm_rope = [&](const uint4 (&raw)[QK_STEPS], const float* gain, uint4 (&res)[QK_STEPS]) {
+            float x[QK_STEPS][8];
+            float ss = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) {
+                const uint32_t w4[4] = {raw[kk].x, raw[kk].y, raw[kk].z, raw[kk].w};
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    x[kk][2 * t] = __uint_as_float(w4[t] << 16);
+                    x[kk][2 * t + 1] = __uint_as_float(w4[t] & 0xffff0000u);
+                    ss += x[kk][2 * t] * x[kk][2 * t] + x[kk][2 * t + 1] * x[kk][2 * t + 1];
+                }
+            }
+            if (gain) {
+                ss = sum_xor32(sum_xor16(ss));
+                const float inv = 1.0f / sqrtf(ss / (float)D + fz.eps);
+#pragma unroll
+                for (int kk = 0; kk < QK_STEPS; ++kk) {
+                    float gn[8];
+                    VecLoad<float, 8>::load(gain + kk * 32 + kb * 8, gn);
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) x[kk][t] = x[kk][t] * inv * gn[t];
+                }
+            }
+            if (fz.rope_table) {
+                constexpr int HK = QK_STEPS / 2;
+#pragma unroll
+                for (int kk = 0; kk < HK; ++kk)
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        const float cs = rope_cs[wave][kk * 32 + kb * 8 + t], sn = rope_cs[wave][D / 2 + kk * 32 + kb * 8 + t];
+                        const float a = x[kk][t], b = x[kk + HK][t];
+                        x[kk][t] = a * cs - b * sn;
+                        x[kk + HK][t] = b * cs + a * sn;
+                    }
+            }
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk)
+                res[kk] = make_uint4(pack_bf16x2(x[kk][0], x[kk][1]), pack_bf16x2(x[kk][2], x[kk][3]),
+                                     pack_bf16x2(x[kk][4], x[kk][5]), pack_bf16x2(x[kk][6], x[kk][7]));
+        };
+        uint4 qn[QK_STEPS];
+        norm_rope(qraw, fz.q_gain, qn);
+#pragma unroll
+        for (int kk = 0; kk < QK_STEPS; ++kk) qf[0][kk] = ok ? qn[kk] : make_uint4(0u, 0u, 0u, 0u);
+        if (own_key && covers) {                              // uniform over the wave
+            uint4 kn[QK_STEPS];
+            norm_rope(kraw, fz.k_gain, kn);
+            if (li == 0) {
+#pragma unroll
+                for (int kk = 0; kk < QK_STEPS; ++kk) new_kv[wave][kk * 4 + kb] = kn[kk];
+            }
+            if (lane < D / 8) new_kv[wave][D / 8 + lane] = vraw;
+            if (chunk == 0) {
+                // to the page, for the steps to come (nothing of this launch reads it there)
+                const int page_i = bs_shift >= 0 ? pos0 >> bs_shift : pos0 / BS;
+                const size_t off = (size_t)table[page_i] * Hkv * BS * D + (size_t)kvh * BS * D +
+                                   (size_t)(pos0 - page_i * BS) * D;
+                if (li == 0) {
+#pragma unroll
+                    for (int kk = 0; kk < QK_STEPS; ++kk)
+                        *reinterpret_cast<uint4*>(fz.k_pool_w + off + kk * 32 + kb * 8) = kn[kk];
+                }
+                if (lane < D / 8) *reinterpret_cast<uint4*>(fz.v_pool_w + off + lane * 8) = vraw;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 
     f32x4_t o[RT][DV];
@@ -467,8 +590,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     // weights, packed as operand B of the second product. The second half is one piece of code
     // behind both variants, so that the accumulators have one home (with the products inside
     // the variants the compiler copies accumulators at every join).
+    // MASKED: keys outside [lo, hi) are not there (their data become zeros), and a row sees
+    // the keys from lo_seen on, up to its own position, inside its window.
     auto scores = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE], auto masked_tag,
-                      s16x4_t (&pf)[RT], float (&alpha)[RT], bool& any_rescale) {
+                      s16x4_t (&pf)[RT], float (&alpha)[RT], bool& any_rescale, int lo, int hi, int lo_seen) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         // V tile -> LDS, row-major with a padded stride (two 8-byte stores per chunk); keys
         // that were not to be read become zeros here, now that their loads have landed
@@ -480,7 +605,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 uint4 t = vr[j];
                 if constexpr (MASKED) {
                     const int vkey = key0 + vk;
-                    if (vkey < kmin || vkey >= khi) t = make_uint4(0u, 0u, 0u, 0u);
+                    if (vkey < lo || vkey >= hi) t = make_uint4(0u, 0u, 0u, 0u);
                 }
                 uint2* dst = reinterpret_cast<uint2*>(&vl[vk * V_STRIDE + part * 8]);
                 dst[0] = make_uint2(t.x, t.y);
@@ -488,7 +613,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             }
         }
         __builtin_amdgcn_wave_barrier();
-        const bool k_ok = !MASKED || (key0 + li >= kmin && key0 + li < khi);
+        const bool k_ok = !MASKED || (key0 + li >= lo && key0 + li < hi);
         any_rescale = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -503,7 +628,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 sv[r] = s[r];
                 if constexpr (MASKED) {
                     const int key = key0 + 4 * kb + r;
-                    bool seen = key <= row_pos[rt] && key < khi && key >= split * split_len;
+                    bool seen = key <= row_pos[rt] && key < hi && key >= lo_seen;
                     if (window > 0) seen = seen && key > row_pos[rt] - window;
                     sv[r] = seen ? sv[r] : -INFINITY;
                 }
@@ -556,10 +681,10 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         float alpha[RT];
         bool any_rescale;
         if constexpr (D > 128) {
-            scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale);     // one variant: registers are short at these sizes
+            scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);     // one variant: registers are short at these sizes
         } else {
-            if (whole) scores(key0, kf, vr, std::false_type{}, pf, alpha, any_rescale);
-            else scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale);
+            if (whole) scores(key0, kf, vr, std::false_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);
+            else scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);
         }
         weighted(pf, alpha, any_rescale);
     };
@@ -600,6 +725,23 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         tile(key0 + 32, kf2, vr2);
     }
 
+    if constexpr (FUSED) {
+        if (own_key && covers) {
+            // the token's own key and value, from where the prologue left them: one more tile
+            // whose first key is the only one there
+            KFrag kfn;
+            uint4 vrn[V_PER_LANE];
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kfn.v[kk] = new_kv[wave][kk * 4 + kb];
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) vrn[j] = new_kv[wave][D / 8 + (lane + 64 * j) % (D / 8)];
+            s16x4_t pf[RT];
+            float alpha[RT];
+            bool any_rescale;
+            scores(pos0, kfn, vrn, std::true_type{}, pf, alpha, any_rescale, pos0, pos0 + 1, pos0);
+            weighted(pf, alpha, any_rescale);
+        }
+    }
     // finish: the row sum is spread over the four lanes of the row's column
     float L[RT];
 #pragma unroll
@@ -784,13 +926,14 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     if (tasks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    const FusedQkv fz{};
     const dim3 grid = n_splits > 1 ? dim3((unsigned)tasks, n_splits / 4) : dim3((unsigned)((tasks + 3) / 4), 1);
     int bs_shift = -1;                                           // log2 of the page size if it is a power of two
     if ((BS & (BS - 1)) == 0)
         for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
-        scale, window, split_len, n_splits, group_pad_log2
+        scale, window, split_len, n_splits, group_pad_log2, fz
     // Row tiles beyond what the registers hold at this head size are refused: two up to head
     // size 128, four up to 64.
     const bool tp = bs_shift >= 4;
@@ -813,6 +956,59 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
 #undef SOC_MFMA_LAUNCH
 #undef SOC_MFMA_ARGS
     return soc_last_error();
+}
+
+
+// A decode step's attention from the QKV product's raw rows (the FUSED form of the kernel
+// above): qkv [N, row_heads, D] with row_heads = Hq + 2 Hkv if write_kv, else at least Hq;
+// q_gain, k_gain [D] float32 or both null; rope_table [rope_positions][2][D / 2] float32
+// (soc_rope_table; every position of the step lies below rope_positions, which the caller
+// checks) or null (no rotation; else it is over the whole head); every token alone. With write_kv the token's key and value
+// are stored at its position in the pools. Head sizes in steps of 32, with a rotation in
+// steps of 64 (returns hipErrorNotSupported otherwise: the caller then runs the kernels one
+// after the other).
+SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, void* k_pool, void* v_pool,
+                                                const int* block_table, int table_width,
+                                                const int* token_rows, const int* positions, void* out,
+                                                float* part_o, float* part_ml, int* arrivals, int N, int Hq,
+                                                int Hkv, int BS, float scale, int window, int split_len,
+                                                int n_splits, int group_pad_log2, const float* q_gain,
+                                                const float* k_gain, const float* rope_table, float eps,
+                                                int write_kv, hipStream_t stream) {
+    if constexpr (!QK_K32) {
+        return (int)hipErrorNotSupported;
+    } else {
+        if (N <= 0) return 0;
+        if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
+            return (int)hipErrorInvalidValue;
+        if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;
+        if (n_splits > 4 && (!part_o || !part_ml || !arrivals)) return (int)hipErrorInvalidValue;
+        if (n_splits > 256 || !(scale > 0.f)) return (int)hipErrorInvalidValue;
+        if ((q_gain == nullptr) != (k_gain == nullptr)) return (int)hipErrorInvalidValue;
+        if (rope_table && D % 64) return (int)hipErrorNotSupported;    // partners of a pair in one lane
+        if (row_heads < (write_kv ? Hq + 2 * Hkv : Hq)) return (int)hipErrorInvalidValue;
+        const int G = Hq / Hkv;
+        if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
+        const long tasks = (long)N * Hkv * ((G + 15) / 16);
+        if (tasks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+        FusedQkv fz{};
+        fz.qkv = (const bf16*)qkv; fz.row_heads = row_heads; fz.q_gain = q_gain; fz.k_gain = k_gain;
+        fz.rope_table = rope_table; fz.eps = eps; fz.write_kv = write_kv ? 1 : 0;
+        fz.k_pool_w = (bf16*)k_pool; fz.v_pool_w = (bf16*)v_pool;
+        const dim3 grid = n_splits > 1 ? dim3((unsigned)tasks, n_splits / 4) : dim3((unsigned)((tasks + 3) / 4), 1);
+        int bs_shift = -1;
+        if ((BS & (BS - 1)) == 0)
+            for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
+#define SOC_FUSED_ARGS (const bf16*)nullptr, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
+        token_rows, positions, (const int*)nullptr, N, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
+        scale, window, split_len, n_splits, group_pad_log2, fz
+        if (bs_shift >= 4)
+            hipLaunchKernelGGL((paged_attn_mfma_kernel<1, true, true>), grid, dim3(256), 0, stream, SOC_FUSED_ARGS);
+        else
+            hipLaunchKernelGGL((paged_attn_mfma_kernel<1, false, true>), grid, dim3(256), 0, stream, SOC_FUSED_ARGS);
+#undef SOC_FUSED_ARGS
+        return soc_last_error();
+    }
 }
 
 

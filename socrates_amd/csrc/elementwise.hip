@@ -650,3 +650,27 @@ SOC_EXPORT int soc_kv_write(const void* k, const void* v, void* k_pool, void* v_
                            token_rows, positions, Hkv, D, BS);
     return soc_last_error();
 }
+
+// ---------------------------------------------------------------------------------------------
+// The rotation's cosines and sines by position, with the arithmetic of the kernels above
+// (float32 angle position * inv_freq, sincosf): out [n_pos][2][half], cosines then sines.
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, int half, int first_pos, int n_pos,
+                                  float* __restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)n_pos * half) return;
+    const int p = (int)(i / half), j = (int)(i % half);
+    float sn, cs;
+    sincosf((float)(first_pos + p) * inv_freq[j], &sn, &cs);
+    out[((size_t)p * 2) * half + j] = cs;
+    out[((size_t)p * 2 + 1) * half + j] = sn;
+}
+
+SOC_EXPORT int soc_rope_table(const float* inv_freq, int half, int first_pos, int n_pos, float* out,
+                              hipStream_t stream) {
+    if (n_pos <= 0) return 0;
+    if (half < 1 || first_pos < 0) return (int)hipErrorInvalidValue;
+    const size_t total = (size_t)n_pos * half;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, inv_freq,
+                       half, first_pos, n_pos, out);
+    return soc_last_error();
+}

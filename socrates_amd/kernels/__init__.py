@@ -45,6 +45,7 @@ _EW_SIGNATURES = {
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
     "soc_rope": [P, P, P, I, I, I, I, I, P],
     "soc_kv_write": [P] * 5 + [I, P, P, I, I, I, I, I, P],
+    "soc_rope_table": [P, I, I, I, P, P],
 }
 _GEMM_SIGNATURES = {
     "soc_gemm_generic": [P, P, P, I, I, I, I, I, I, P],
@@ -59,6 +60,7 @@ _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
+    "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, P],
     "soc_attention_head_dim": [],
 }
 
@@ -138,6 +140,8 @@ class HipKernels:
         # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
         self.fuse_norms = True
+        # decode steps: per-head norm, rotation and the page write inside the attention kernel
+        self.fuse_rope = True
         self.addnorm_waves = 0          # waves of such a projection, override
         self.addnorm_splits = 0         # workgroups that share one tile's K in it, override
         # arrival counts of those workgroups, one per tile of 16 outputs: zero between launches
@@ -624,6 +628,73 @@ class HipKernels:
             c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(self._split_count), c_int(N),
             c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
             c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
+
+    def rope_table(self, inv_freq, first_pos, n_pos, out=None):
+        """Cosines and sines of positions first_pos .. first_pos + n_pos - 1 with the rotation
+        kernels' own arithmetic: float32 [n_pos, 2, len(inv_freq)] (into ``out`` if given)."""
+        half = inv_freq.numel()
+        self._want(inv_freq, "inv_freq", torch.float32, (half,))
+        if out is None:
+            out = torch.empty((n_pos, 2, half), dtype=torch.float32, device=self.device)
+        self._want(out, "table", torch.float32, (n_pos, 2, half))
+        _check(self._ew.soc_rope_table(_ptr(inv_freq), c_int(half), c_int(first_pos), c_int(n_pos), _ptr(out),
+                                       self._stream()), "rope_table")
+        return out
+
+    def decode_attention(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps, rope_table, slot, ctx, scale,
+                         window=None, write=True):
+        """A decode step's attention straight from the QKV product's rows: per-head norm,
+        rotation, the write of the new key and value, and the attention over the pages in one
+        kernel. ``qkv`` [N, (Hq + 2 Hkv) D] (with ``write``) or [N, Hq D]. Returns [N, Hq D],
+        or None where this form does not apply (the caller then runs the kernels one after
+        the other): bfloat16 steps in which every request brings one token, head sizes in
+        steps of 32 without a rotation, in steps of 64 with one (``rope_table``, over the whole
+        head: a lane's slices of a head then hold both partners of every rotated pair)."""
+        if not (self.fuse_rope and self.dtype == torch.bfloat16 and self.attention_mfma
+                and getattr(ctx, "max_q_len", 0) == 1 and D % 32 == 0 and 32 <= D <= 256
+                and (rope_table is None or D % 64 == 0) and slot is not None):
+            return None
+        N = qkv.shape[0]
+        heads = Hq + 2 * Hkv if write else Hq
+        if N > 65535 or Hq % Hkv:
+            return None
+        self._want(qkv, "qkv", self.dtype, (N, heads * D))
+        if (q_gain is None) != (k_gain is None):
+            raise KernelError("q and k gains come together")
+        if q_gain is not None:
+            self._want(q_gain, "q gain", torch.float32, (D,))
+            self._want(k_gain, "k gain", torch.float32, (D,))
+        if rope_table is not None:
+            # [positions, 2, D / 2] from ``rope_table``, a rotation over the whole head; every
+            # position of the step must lie in it
+            self._want(rope_table, "rope table", torch.float32, (rope_table.shape[0], 2, D // 2))
+            if rope_table.shape[0] < ctx.max_ctx_len:
+                raise KernelError(f"the rotation's table holds {rope_table.shape[0]} positions, the step "
+                                  f"reaches {ctx.max_ctx_len}")
+        self._check_slot(slot, Hkv, D)
+        self._want(ctx.positions, "positions", torch.int32, (N,))
+        self._want(ctx.token_rows, "token_rows", torch.int32, (N,))
+        lib = self._attention_lib(D)
+        G = Hq // Hkv
+        gpl = max(0, (min(G, 16) - 1).bit_length())
+        split_len, n_splits = self.plan_mfma(N, Hkv, G, ctx.max_ctx_len)
+        part_o = part_ml = None
+        if n_splits > 4:
+            tasks = N * Hkv * ((G + 15) // 16)
+            if tasks > self._split_count.numel():
+                return None
+            part_o = torch.empty((N, Hq, n_splits // 4, D), dtype=torch.float32, device=self.device)
+            part_ml = torch.empty((N, Hq, n_splits // 4, 2), dtype=torch.float32, device=self.device)
+        out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
+        self.last_attention_kernel = ("fused", 1)
+        _check(lib.soc_paged_attention_decode_fused(
+            _ptr(qkv), c_int(heads), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
+            c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(out), _ptr(part_o),
+            _ptr(part_ml), _ptr(self._split_count), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
+            c_float(scale), c_int(int(window) if window else 0), c_int(split_len), c_int(n_splits), c_int(gpl),
+            _ptr(q_gain), _ptr(k_gain), _ptr(rope_table), c_float(eps), c_int(1 if write else 0), self._stream()),
+            "decode_attention")
+        return out
 
     def paged_attention(self, q, slot, ctx, scale, window=None):
         """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""

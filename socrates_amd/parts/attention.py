@@ -63,7 +63,16 @@ class PagedAttention:
             qkv = ops.linear(x, self.w_qkv[: Hq * D])
             Hkv = 0
         rot = self.position.rotary() if hasattr(self.position, "rotary") else None
-        if self.position is None or rot is not None:
+        o = None
+        if (self.position is None or rot is not None) and hasattr(ops, "decode_attention"):
+            # a decode step: norm, position encoding, cache write and attention in one kernel
+            table = self.position.table(ctx.max_ctx_len) if hasattr(self.position, "table") else None
+            if self.position is None or table is not None:
+                o = ops.decode_attention(qkv, Hq, s.n_kv_heads, D, self.q_gain, self.k_gain, self.eps, table,
+                                         slot, ctx, s.scale, s.window, write)
+        if o is not None:
+            pass
+        elif self.position is None or rot is not None:
             inv_freq, rotary_dim = rot if rot is not None else (None, 0)
             q = ops.qk_norm_rope_write(
                 qkv, Hq, Hkv, D, self.q_gain, self.k_gain, self.eps, inv_freq, rotary_dim,
@@ -74,7 +83,8 @@ class PagedAttention:
             self.position.apply(q, k, ctx.positions)
             if write:
                 ops.kv_write(k, v, ctx.positions, ctx.token_rows, slot)
-        o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
+        if o is None:
+            o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
         if project is not None:
             return project(o, self.w_o)
         # the block's next norm adds this output to the residual: partial sums are welcome

@@ -298,6 +298,67 @@ def test_paged_attention_decode_tokens(kernel_sets, dtype, Hq, Hkv, D, bs):
     hip.attention_splits = None
 
 
+@pytest.mark.parametrize("Hq,Hkv,D,bs,norm,rope", [(32, 8, 128, 16, True, True), (16, 1, 64, 32, True, True),
+                                                   (8, 2, 32, 8, True, False), (6, 3, 128, 4, False, True),
+                                                   (2, 1, 256, 16, True, True), (40, 2, 64, 12, False, False),
+                                                   (5, 5, 96, 2, True, False)])
+def test_decode_attention_from_raw_qkv(kernel_sets, Hq, Hkv, D, bs, norm, rope):
+    """A decode step's attention in one kernel (per-head norm, rotation, the new key and value,
+    the walk over the pages) against the kernels one after the other, and against plain
+    attention on what those wrote: lengths at page and tile edges (a first token, a new page,
+    a full tile), with and without key splits, window, norm and rotation. The page slot of the
+    new token holds poison before the call and the new key and value after it."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    lens = [1, 15, 16, 17, 33, 300, 1025]
+    N = len(lens)
+    rows, pos = list(range(N)), [n - 1 for n in lens]
+    q_gain = (1 + 0.3 * torch.randn(D)).to(DEV) if norm else None
+    k_gain = (1 + 0.3 * torch.randn(D)).to(DEV) if norm else None
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV) if rope else None
+    qkv = rnd((N, (Hq + 2 * Hkv) * D), torch.bfloat16, 60, 1.5)
+    ctx = ctx_for(rows, pos)
+    table = None
+    if rope:
+        # the table in two pieces, as a part grows it; it holds what an accurate sincosf gives
+        table = torch.empty((1100, 2, D // 2), dtype=torch.float32, device=DEV)
+        hip.rope_table(inv_freq, 0, 300, table[:300])
+        hip.rope_table(inv_freq, 300, 800, table[300:])
+        ang = torch.arange(1100, dtype=torch.float32)[:, None] * inv_freq.cpu()[None]
+        torch.testing.assert_close(table[:, 0].cpu(), ang.double().cos().float(), atol=2e-6, rtol=0)
+        torch.testing.assert_close(table[:, 1].cpu(), ang.double().sin().float(), atol=2e-6, rtol=0)
+    for window in (None, 40):
+        for splits in (None, (64, 17), (16, 256), (1 << 30, 1)):
+            hip.attention_splits = splits
+            slot_a, _ = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=D + 2)
+            slot_b, _ = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=D + 2)
+            for slot in (slot_a, slot_b):               # poison where the new tokens go
+                for r, p_ in zip(rows, pos):
+                    page = int(slot.block_table[r, p_ // bs])
+                    slot.k[page, :, p_ % bs] = float("nan")
+                    slot.v[page, :, p_ % bs] = float("inf")
+            hip.fuse_rope = False
+            q = hip.qk_norm_rope_write(qkv, Hq, Hkv, D, q_gain, k_gain, 1e-6, inv_freq, D if rope else 0,
+                                       ctx.positions, ctx.token_rows, slot_a)
+            want = hip.paged_attention(q, slot_a, ctx, 0.2, window)
+            hip.fuse_rope = True
+            got = hip.decode_attention(qkv, Hq, Hkv, D, q_gain, k_gain, 1e-6, table, slot_b, ctx, 0.2, window, True)
+            assert got is not None and hip.last_attention_kernel == ("fused", 1)
+            close(got, want, torch.bfloat16)
+            # the pages: values exact, keys to a rounding of bfloat16 (the sum of squares is added in another order)
+            assert torch.equal(slot_b.v, slot_a.v)
+            torch.testing.assert_close(slot_b.k.float(), slot_a.k.float(), atol=2e-2, rtol=1e-2)
+            # reading only (another layer wrote the slot): queries from a row without k and v heads
+            got_r = hip.decode_attention(qkv[:, :Hq * D].contiguous(), Hq, Hkv, D, q_gain, k_gain, 1e-6, table,
+                                         slot_a, ctx, 0.2, window, False)
+            close(got_r, want, torch.bfloat16)
+    hip.attention_splits = None
+    assert int(hip._split_count.abs().sum()) == 0
+    # where the form does not apply the caller is told so
+    assert hip.decode_attention(qkv[:, :(Hq + 2 * Hkv) * 16], Hq, Hkv, 16, None, None, 1e-6, None, slot_a, ctx, 0.2) is None
+    table32 = torch.zeros((1100, 2, 16), device=DEV)      # a rotation at head size 32: partners lie in different lanes
+    assert hip.decode_attention(qkv[:, :(Hq + 2 * Hkv) * 32], Hq, Hkv, 32, None, None, 1e-6, table32, slot_a, ctx, 0.2) is None
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     """Tokens of one row at consecutive positions (a portion that starts mid-sequence)
