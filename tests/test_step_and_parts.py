@@ -469,3 +469,71 @@ def test_a_toy_routed_feed_forward_and_a_toy_position_encoding(kind, dtype):
     x = plain.block(x, w, 1, cfg, pos)
     want = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
     torch.testing.assert_close(outs[0], want, **tol)
+
+
+@dataclass(frozen=True)
+class ReluSpec:
+    """y = Down(relu(Up x)): a feed-forward that opts into the block's folded sums and norms."""
+    hidden: int
+    intermediate: int
+
+
+class ReluFeedForward:
+    takes_projection = True     # ends with a projection the block may supply
+    takes_norm_owed = True      # hands x to one product only
+
+    @staticmethod
+    def tensors(spec):
+        return {"up.weight": TensorDecl((spec.intermediate, spec.hidden)),
+                "down.weight": TensorDecl((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec, tensors, ops):
+        self.ops, self.t = ops, tensors
+        self.calls = []
+
+    def forward(self, x, ctx=None, project=None):
+        self.calls.append((type(x).__name__, project is not None))
+        h = torch.relu(self.ops.linear(x, self.t["up.weight"]))
+        if project is not None:
+            return project(h, self.t["down.weight"])
+        return self.ops.linear(h, self.t["down.weight"], allow_partial=True)
+
+
+@pytest.mark.gpu
+def test_a_toy_feed_forward_takes_the_blocks_folded_sums_and_norms():
+    """A part defined here opts into the two optional attributes and gets, in short bfloat16
+    steps, rows that are still owed their norm and a projection that adds to the residual
+    stream itself; in long steps and with the folding switched off it gets plain tensors. The
+    logits agree either way, and with a whole-prompt run."""
+    register_part(ReluSpec, ReluFeedForward)
+    ops = kernels("hip", torch.bfloat16)
+    hidden = 64
+    att = AttentionSpec(hidden, 4, 2, 16, 16 ** -0.5, RMSNormSpec(16, 1e-6), RopeSpec(16, 1e4))
+    blocks = [BlockSpec(att, ReluSpec(hidden, 96), RMSNormSpec(hidden, 1e-6), RMSNormSpec(hidden, 1e-5),
+                        prefix=f"model.layers.{i}.") for i in range(3)]
+    plan = plan_with(blocks, [RunStep(0, 0), RunStep(1, 1), RunStep(2, 2)], hidden)
+    tokens = random_prompts([40], 50, seed=4)[0]
+    weights = random_tensors(expected_tensors(plan), seed=3, dtype=ops.dtype, device=ops.device, std=0.2, gain_std=0.1)
+    results, seen = {}, {}
+    for fused in (True, False):
+        ops.fuse_norms = fused
+        model = DecoderModel(plan, weights, ops)
+        cache = CacheManager(cache_needs(plan), 2, 64, 8, 16, ops.dtype, ops.device)
+        runner = ModelRunner(model, cache)
+        row = cache.open_row()
+        logits, t = [], 0
+        for n in [20, 3, 1, 1, 14, 1]:
+            logits.append(runner.step([StepEntry(row, tokens[t:t + n], list(range(n)))]).float().cpu())
+            t += n
+        results[fused] = torch.cat(logits)
+        seen[fused] = model.blocks[1].ffn.calls
+    ops.fuse_norms = True
+    # the long first step: plain rows in, yet the projection is the block's (it runs product, sum
+    # and norm one after the other); short steps: rows owed their norm
+    assert seen[True][0] == ("Tensor", True) and seen[True][1] == ("NormOwed", True)
+    assert all(kind == "Tensor" for kind, _ in seen[False])
+    torch.testing.assert_close(results[True], results[False], atol=0.1, rtol=5e-2)
+    model = DecoderModel(plan, weights, ops)
+    cache = CacheManager(cache_needs(plan), 2, 64, 8, 16, ops.dtype, ops.device)
+    whole_run = ModelRunner(model, cache).step([StepEntry(cache.open_row(), tokens, list(range(40)))]).float().cpu()
+    torch.testing.assert_close(results[True], whole_run, atol=0.1, rtol=5e-2)
