@@ -337,6 +337,11 @@ class HipKernels:
             tunable.enable(True)
             tunable.set_max_tuning_duration(30)          # ms per solution
             tunable.set_max_tuning_iterations(20)
+            # Only solutions that agree with the library's default to a rounding of bfloat16 are
+            # candidates: some of the faster ones round more often on the way (measured: logits
+            # of a tiny model off by twice the usual error when one of them had been picked),
+            # and which one is fastest varies from run to run.
+            tunable.set_numerical_check_tolerances(True, 1e-3, 8e-3)
         tunable.tuning_enable(bool(on))
         self._tuning = bool(on)
         if not on:

@@ -76,12 +76,13 @@ def test_temperature_tiny_b_workload(tmp_path):
             ids.append(tok)
 
 
-def test_tuned_library_products_leave_the_tokens_alone(tmp_path):
+def test_tuned_library_products_leave_the_tokens_alone(tmp_path, request):
     """``Engine.tune``: the library picks its fastest solution for the products of a 33-token
     portion (bfloat16, more than 16 rows); greedy tokens stay those of the plain run, the
     counters and the cache are as before, and nothing is written to the working folder."""
     import os
     from socrates_amd.engine import Engine
+    request.addfinalizer(lambda: torch.cuda.tunable.enable(False))     # what is tuned here stays here
     folder = write_tiny(tmp_path / "A", TINY_A, seed=0)
     cfg, w = plain.read_folder(folder, torch.float64)
     prompts = random_prompts([33, 20], cfg["vocab_size"], seed=3)
