@@ -202,6 +202,8 @@ def main(argv=None):
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-tune", action="store_true", help="library products with the library's default choice")
+    ap.add_argument("--split-waves", type=int, default=None, help="key splits of the decode attention: waves aimed at")
+    ap.add_argument("--split-keys", type=int, default=None, help="key splits of the decode attention: fewest keys of a split")
     ap.add_argument("--no-fused-norms", action="store_true",
                     help="decode steps with the residual sums and norms in kernels of their own")
     args = ap.parse_args(argv)
@@ -228,6 +230,10 @@ def main(argv=None):
     config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
     V = config.vocab_size
     engine.runner.ops.fuse_norms = not args.no_fused_norms
+    if args.split_waves:
+        engine.runner.ops.split_target_waves = args.split_waves
+    if args.split_keys:
+        engine.runner.ops.split_min_keys = args.split_keys
     if args.dtype == "bf16" and not args.no_tune:
         # the library's products (more than 16 rows): its fastest solution for the prompt's shapes
         # and, up to 16 rows, the faster of the library and this package's own kernel for the timed batch

@@ -366,7 +366,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        const int* __restrict__ positions, const int* __restrict__ row_blocks,
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
                        float* __restrict__ part_ml, int* __restrict__ arrivals, int Hq, int Hkv, int BS,
-                       int bs_shift, float scale, int window, int split_len, int n_splits,
+                       int bs_shift, float scale, int window, int split_len_arg, int n_splits,
                        int group_pad_log2, FusedQkv fz) {
     static_assert(!FUSED || (RT == 1 && QK_K32), "the fused form: one row tile, head sizes in steps of 32");
     // One piece of LDS: the waves' V tiles while the keys are walked; afterwards, with key
@@ -397,7 +397,16 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     const int* table = block_table + (size_t)token_rows[tok0] * table_width;
 
     // keys this wave walks: its split, cut to what its rows can see
-    int klo = split * split_len;
+    // split_len_arg 0: the keys this block's rows can see are shared out evenly among the
+    // n_splits waves of the task (whole tiles of 16), whatever length the launch was planned
+    // for: no wave of a short row walks far, none of a long row is idle
+    int split_len = split_len_arg, first_key = 0;
+    if (split_len_arg <= 0) {
+        first_key = window > 0 ? max(0, pos0 - window + 1) & ~15 : 0;
+        split_len = max(16, ((pos0 + ntok - first_key + n_splits - 1) / n_splits + 15) & ~15);
+    }
+    const int split_lo = first_key + split * split_len;     // the split's first key
+    int klo = split_lo;
     // FUSED and writing: the token's own key is not read from the cache (it is not there yet)
     const bool own_key = FUSED && fz.write_kv;
     const bool covers = pos0 >= klo && pos0 < klo + split_len;      // this wave's split holds the token's position
@@ -675,16 +684,16 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     // and inside the window of its last one, so no score needs a mask
     const int last_pos = pos0 + ntok - 1;
     auto tile = [&](int key0, const KFrag& kf, const uint4 (&vr)[V_PER_LANE]) {
-        const bool whole = key0 >= split * split_len && key0 + 15 < khi && key0 + 15 <= pos0 &&
+        const bool whole = key0 >= split_lo && key0 + 15 < khi && key0 + 15 <= pos0 &&
                            (window <= 0 || key0 > last_pos - window);
         s16x4_t pf[RT];
         float alpha[RT];
         bool any_rescale;
         if constexpr (D > 128) {
-            scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);     // one variant: registers are short at these sizes
+            scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split_lo);     // one variant: registers are short at these sizes
         } else {
-            if (whole) scores(key0, kf, vr, std::false_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);
-            else scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split * split_len);
+            if (whole) scores(key0, kf, vr, std::false_type{}, pf, alpha, any_rescale, kmin, khi, split_lo);
+            else scores(key0, kf, vr, std::true_type{}, pf, alpha, any_rescale, kmin, khi, split_lo);
         }
         weighted(pf, alpha, any_rescale);
     };
@@ -901,7 +910,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 // (16 * row_tiles) >> group_pad_log2 tokens of one sequence, or null: every token is a block
 // of its own (n_row_blocks = N); 2^group_pad_log2 >= min(G, 16).
 // Splits are over absolute key indices: split s covers keys [s * split_len, (s + 1) * split_len),
-// split_len a multiple of 16. n_splits > 1 must be a multiple of 4 (four splits share a
+// split_len a multiple of 16; or split_len 0: every row block's visible keys are shared out
+// evenly among its n_splits splits (whole tiles of 16). n_splits > 1 must be a multiple of 4 (four splits share a
 // workgroup), at most 256, and needs part_o [R, Hq, n_splits / 4, D] and part_ml
 // [R, Hq, n_splits / 4, 2] if n_splits > 4, with R = N without row blocks, else n_row_blocks *
 // tokens per block (the blocks may cover some of the N tokens only; the others' outputs are
@@ -915,7 +925,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
                                         int Hq, int Hkv, int BS, float scale, int window, int split_len,
                                         int n_splits, int row_tiles, int group_pad_log2, hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
-    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
+    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
         return (int)hipErrorInvalidValue;
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;
@@ -979,7 +989,7 @@ SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, 
         return (int)hipErrorNotSupported;
     } else {
         if (N <= 0) return 0;
-        if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 16 || split_len % 16)
+        if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
             return (int)hipErrorInvalidValue;
         if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;
         if (n_splits > 4 && (!part_o || !part_ml || !arrivals)) return (int)hipErrorInvalidValue;

@@ -74,7 +74,7 @@ def _declare(lib, signatures):
 MAX_KEY_SPLITS = 256    # of the MFMA attention: 64 workgroups of four splits meet per task
 
 
-def plan_key_splits(n_blocks, n_kv_heads, group, max_keys):
+def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, min_keys=64):
     """(split_len, n_splits) for the MFMA attention kernel: enough waves to fill the GPU, no
     split shorter than 64 keys, at most MAX_KEY_SPLITS of them (a longer context gets longer
     splits), one split or a multiple of four (four share a workgroup; some of the last four
@@ -82,8 +82,8 @@ def plan_key_splits(n_blocks, n_kv_heads, group, max_keys):
     16 keys long, and cover keys 0 .. max_keys - 1. Host arithmetic only."""
     waves = n_blocks * n_kv_heads * ((group + 15) // 16)
     # from one wave per SIMD on (1,024) no split: a split costs a trip through LDS, or memory
-    n = 1 if waves >= 1024 else max(1, min((2048 + waves - 1) // waves, (max_keys + 63) // 64,
-                                           MAX_KEY_SPLITS))
+    n = 1 if waves >= 1024 else max(1, min((target_waves + waves - 1) // waves,
+                                           (max_keys + min_keys - 1) // min_keys, MAX_KEY_SPLITS))
     if n == 1:
         return ((max_keys + 15) // 16 * 16), 1
     n = (n + 3) // 4 * 4
@@ -142,6 +142,12 @@ class HipKernels:
         self.fuse_norms = True
         # decode steps: per-head norm, rotation and the page write inside the attention kernel
         self.fuse_rope = True
+        # key splits of the MFMA decode attention: waves aimed at, and the fewest keys of a split
+        # (measured at 8 kv heads of 128, context 2,048, in ms per step of a 4B-sized model at
+        # 1,024 / 2,048 / 4,096 waves: batch 4: 2.92 / 2.97 / 2.97; 8: 3.36 / 3.41 / 3.59; 16:
+        # 4.49 / 4.37 / -; 24: 5.09 / 5.15 / 5.16; 32: 5.32 / 5.51 / 5.57: more splits mean more
+        # workgroups that have to meet in memory)
+        self.split_target_waves, self.split_min_keys = 1024, 64
         self.addnorm_waves = 0          # waves of such a projection, override
         self.addnorm_splits = 0         # workgroups that share one tile's K in it, override
         # arrival counts of those workgroups, one per tile of 16 outputs: zero between launches
@@ -606,7 +612,7 @@ class HipKernels:
                 raise KernelError(f"{n_splits} key splits asked for; the MFMA attention kernel takes at "
                                   f"most {MAX_KEY_SPLITS}")
             return split_len, n_splits
-        return plan_key_splits(n_blocks, n_kv_heads, group, max_keys)
+        return plan_key_splits(n_blocks, n_kv_heads, group, max_keys, self.split_target_waves, self.split_min_keys)
 
     def _wave_attention(self, lib, q, slot, ctx, out, scale, w, rt, gpl, which):
         """The per-wave MFMA kernel with key splits and merge, for all sequences of the step
@@ -617,6 +623,8 @@ class HipKernels:
         tokens_per_block = max(1, (16 * rt) >> gpl)
         blocks, n_blocks = self._row_blocks(ctx, N, tokens_per_block, which)
         split_len, n_splits = self.plan_mfma(n_blocks, Hkv, G, ctx.max_ctx_len)
+        if self.attention_splits is None and n_splits > 1:
+            split_len = 0           # the kernel shares every row's own keys out evenly among the splits
         part_o = part_ml = None
         if n_splits > 4:
             # the workgroups of a task (four splits each) meet in memory
@@ -683,6 +691,8 @@ class HipKernels:
         G = Hq // Hkv
         gpl = max(0, (min(G, 16) - 1).bit_length())
         split_len, n_splits = self.plan_mfma(N, Hkv, G, ctx.max_ctx_len)
+        if self.attention_splits is None and n_splits > 1:
+            split_len = 0           # the kernel shares every row's own keys out evenly among the splits
         part_o = part_ml = None
         if n_splits > 4:
             tasks = N * Hkv * ((G + 15) // 16)
