@@ -285,9 +285,11 @@ __device__ __forceinline__ void sk_ssq_shares(const SkNorm& nm, int M, int wave,
     const int pairs = 16 * ((nm.ssq_tiles + 255) / 256);
 #pragma unroll
     for (int u = 0; u < SK_SSQ_AHEAD; ++u) {
-        const int pair = wave + u * n_waves;
-        const float s = wave_sum(sk_ssq_masked(nm, M, pair, lane, v[u]));
-        if (lane == 0 && pair < pairs && pair < SK_SSQ_MAX_PAIRS) part[pair] = s;
+        const int pair = wave + u * n_waves;                 // the same in all lanes
+        if (pair >= pairs || pair >= SK_SSQ_MAX_PAIRS) continue;
+        // (a row beyond M has no sum to take: nothing reads its place)
+        const float s = pair % 16 < M ? wave_sum(sk_ssq_masked(nm, M, pair, lane, v[u])) : 0.f;
+        if (lane == 0) part[pair] = s;
     }
     for (int pair = wave + SK_SSQ_AHEAD * n_waves; pair < pairs && pair < SK_SSQ_MAX_PAIRS; pair += n_waves) {
         const float s = wave_sum(sk_ssq_masked(nm, M, pair, lane, sk_ssq_load(nm, M, pair, lane)));
