@@ -145,6 +145,7 @@ class Qwen3Config:
             layers=layers, order=default_order(len(layers)), final_norm=norm,
             embedding_name="model.embed_tokens.weight", final_norm_prefix="model.norm",
             head_name=None if self.tie_word_embeddings else "lm_head.weight",
+            duplicates=(("lm_head.weight", "model.embed_tokens.weight"),) if self.tie_word_embeddings else (),
             eos_token_ids=self.eos_token_ids)
 
     # ---- byte and flop counts (analysis/arithmetic.py:75-143) ----------------------------

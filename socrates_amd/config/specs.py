@@ -118,6 +118,9 @@ class ModelPlan:
     final_norm_prefix: str
     head_name: Optional[str]      # None: the head is the embedding table (tied)
     eos_token_ids: Tuple[int, ...] = field(default=())
+    # (stored name, name of an expected tensor): a checkpoint may also store the first if it
+    # holds the very same values as the second (a tied head written out beside the embedding)
+    duplicates: Tuple[Tuple[str, str], ...] = field(default=())
 
     def __post_init__(self):
         written = set()

@@ -42,7 +42,7 @@ class ModelRunner:
         if ops is None:
             from ..kernels import HipKernels
             ops = HipKernels(dtype, device)
-        weights = load_weights(folder, expected_tensors(plan), dtype, device)
+        weights = load_weights(folder, expected_tensors(plan), dtype, device, plan.duplicates)
         model = DecoderModel(plan, weights, ops)
         cache = CacheManager(cache_needs(plan), max_rows=max_rows, max_len=max_len,
                              block_size=block_size, num_blocks=num_blocks, dtype=dtype,

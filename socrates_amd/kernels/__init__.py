@@ -132,6 +132,16 @@ class HipKernels:
         self._tuning = False
         self.attention_mfma = True          # bfloat16 takes the MFMA kernels
         self.attention_workgroup = True     # prompt portions take the kernel that shares K/V through LDS
+        # Which form of the prompt-portion attention a step takes, by the number of workgroups
+        # its long portions give (of 32 rows x 4 waves for the first three, of the chosen form
+        # for the last). Measured on an MI355X (256 compute units) at 8 kv heads of 4 x 128 and
+        # 4 x 64; another head layout or another GPU may want other values: set them here.
+        self.prompt_form_thresholds = {
+            "workgroup_kernel": 256,          # below: the per-wave kernel with key splits
+            "eight_waves": 256,               # from here: 32 rows per wave, keys in two halves
+            "four_waves_of_32_rows": 768,     # from here (head sizes over 64): four waves of 32 rows
+            "two_tiles_of_16_rows": 512,      # head sizes that are no multiple of 32, up to 64
+        }
         # bfloat16 products with more than 16 rows go to the library (hipBLASLt through
         # torch.mm), as the reference's all do (nn.Linear); False keeps them on this
         # package's tiled MFMA kernel
@@ -749,6 +759,7 @@ class HipKernels:
             #   3,072 from 0 (768): 163 / 112 / 107 / 123;  8,192 (2,048): 941 / 650 / 633 / 695
             #   1,024 behind 3,072 (256): 117 / 122 / 111 / 89;  2,048 behind 6,144 (512): 488 / 305 / 296 / 297
             # at head size 64 the eight-wave form stays ahead or level up to 8,192 tokens.
+            th = self.prompt_form_thresholds
             wg_rt = 1
             if self.attention_row_tiles in (1, 2, 32, 64):
                 wg_rt = self.attention_row_tiles
@@ -756,11 +767,11 @@ class HipKernels:
                     wg_rt = 1
             elif D % 32 == 0:
                 n32 = (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16)
-                if n32 >= 768 and D > 64:
+                if n32 >= th["four_waves_of_32_rows"] and D > 64:
                     wg_rt = 32
-                elif n32 >= 256:
+                elif n32 >= th["eight_waves"]:
                     wg_rt = 64
-            elif D <= 64 and (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16) >= 512:
+            elif D <= 64 and (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16) >= th["two_tiles_of_16_rows"]:
                 wg_rt = 2
             wg_tokens = 4 * max(1, (32 if wg_rt >= 32 else 16 * wg_rt) >> gpl)
             # Prompt portions go to the kernel whose four waves share the K and V tiles, if it
@@ -769,7 +780,8 @@ class HipKernels:
             # shorter portion behind a long context is better served by the per-wave kernel
             # with key splits (128 tokens behind 8 k: 95 us against 196 us). An override of
             # the row tiles (tests) forces the choice.
-            enough = (n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= 256 or self.attention_row_tiles is not None
+            enough = ((n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= th["workgroup_kernel"]
+                      or self.attention_row_tiles is not None)
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
                 rt = wg_rt

@@ -77,17 +77,29 @@ def kept_dtype(kind: str, stored: str, compute_dtype):
     return compute_dtype
 
 
-def load_weights(folder, expected, compute_dtype, device):
+def _same_stored(where, a, b) -> bool:
+    """Whether the stored tensors ``a`` and ``b`` hold the same values in the same dtype."""
+    with safe_open(str(where[a]), framework="pt") as fa, safe_open(str(where[b]), framework="pt") as fb:
+        ta, tb = fa.get_tensor(a), fb.get_tensor(b)
+    return ta.dtype == tb.dtype and ta.shape == tb.shape and torch.equal(ta, tb)
+
+
+def load_weights(folder, expected, compute_dtype, device, duplicates=()):
     """Read the tensors named in ``expected`` ({name: TensorDecl}) from ``folder``.
 
     Returns {name: tensor on device}. Raises WeightError naming everything that
     does not fit. As under the reference's strict load, an ``lm_head.weight`` in
-    the folder of a tied model is unexpected.
+    the folder of a tied model is unexpected, unless ``duplicates`` ((stored name,
+    expected name) pairs, ``ModelPlan.duplicates``) names it and it holds the very
+    values of the embedding table; it is then not read.
     """
     folder = Path(folder)
     where = _files_of(folder)
     missing = [n for n in expected if n not in where]
     unexpected = [n for n in where if n not in expected]
+    for stored, same_as in duplicates:
+        if stored in unexpected and same_as in where and _same_stored(where, stored, same_as):
+            unexpected.remove(stored)
     wrong_shape, wrong_dtype = [], []
     by_file = {}
     for name, decl in expected.items():

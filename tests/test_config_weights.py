@@ -197,3 +197,26 @@ def test_sharded_folder_with_index(tmp_path):
                for n in names if t[n].dim() == 2)
     with pytest.raises(FileNotFoundError):
         load_weights(tmp_path, expected_tensors(cfg.plan()), torch.bfloat16, "cpu")
+
+
+def test_a_tied_checkpoint_may_store_its_head_if_it_is_the_embedding_table(tmp_path):
+    """Some exporters write ``lm_head.weight`` beside the embedding although the two are tied:
+    accepted if and only if the values are the same; never loaded twice."""
+    from safetensors.torch import load_file, save_file
+    cfg = Qwen3Config.from_dict(TINY_A["cfg"])
+    plan = cfg.plan()
+    folder = write_random_model(tmp_path / "m", cfg, seed=1)
+    path = folder / "model.safetensors"
+    t = load_file(str(path))
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    save_file(t, str(path))
+    w = load_weights(folder, expected_tensors(plan), torch.bfloat16, "cpu", plan.duplicates)
+    assert "lm_head.weight" not in w and set(w) == set(expected_tensors(plan))
+    with pytest.raises(WeightError) as e:                    # without the plan's say-so it stays unexpected
+        load_weights(folder, expected_tensors(plan), torch.bfloat16, "cpu")
+    assert e.value.unexpected == ["lm_head.weight"]
+    t["lm_head.weight"][3, 5] += 1
+    save_file(t, str(path))
+    with pytest.raises(WeightError) as e:
+        load_weights(folder, expected_tensors(plan), torch.bfloat16, "cpu", plan.duplicates)
+    assert e.value.unexpected == ["lm_head.weight"]
