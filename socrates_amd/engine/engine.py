@@ -24,10 +24,18 @@ from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
 from .request import MAX_BATCH, MAX_LEN, MAX_NEW_TOKENS, MAX_QUEUE, QueueFull, Request, TooLong  # noqa: F401
 from .runner import ModelRunner
-from .scheduler import Scheduler
+from .scheduler import Planned, Scheduler
 
 KV_BLOCK = 16          # model/inference_paged.py:51
 PREFILL_CHUNK = 2048   # token budget of one step
+
+
+class _Flight:
+    """A step that is queued on the device and whose tokens have not been taken yet."""
+    __slots__ = ("plan", "wanted", "drawn")
+
+    def __init__(self, plan, wanted, drawn):
+        self.plan, self.wanted, self.drawn = plan, wanted, drawn
 
 
 class Engine:
@@ -35,7 +43,7 @@ class Engine:
                  compile: bool = True, max_batch: int = MAX_BATCH, max_len: int = MAX_LEN,
                  max_new_tokens: int = MAX_NEW_TOKENS, block_size: int = KV_BLOCK,
                  num_blocks: Optional[int] = None, chunk: int = PREFILL_CHUNK,
-                 max_queue: int = MAX_QUEUE, template=None):
+                 max_queue: int = MAX_QUEUE, template=None, lookahead: bool = True):
         """model: a model folder (config.json + safetensors) or a ModelRunner. tok: an
         optional tokenizer with the HF surface the reference uses (``apply_chat_template``,
         ``__call__``, ``all_special_ids``); without one, prompts are token id lists.
@@ -43,7 +51,9 @@ class Engine:
         pool; default is the worst case max_batch * ceil(max_len / block_size)
         (model/inference_paged.py:83-84). template: ``template(tok, text) -> token ids`` for
         text prompts; default: what the model's configuration class offers as
-        ``chat_prompt`` (the architecture's chat format), else the tokenizer's plain encoding."""
+        ``chat_prompt`` (the architecture's chat format), else the tokenizer's plain encoding.
+        lookahead: queue the next decode step before the last one's tokens are read (see
+        ``step``); it needs ``compile``."""
         self.device, self.max_batch = device, max_batch
         self.max_len, self.max_new_tokens = max_len, max_new_tokens
         self.tok = tok
@@ -62,6 +72,9 @@ class Engine:
         self.compile = compile
         if compile and hasattr(self.runner, "enable_graphs"):
             self.runner.enable_graphs(max_batch)
+        self.lookahead = bool(lookahead and compile and hasattr(self.runner, "feeds"))
+        self._flight: Optional[_Flight] = None   # the step queued ahead, if any
+        self.n_ahead = 0                # steps that were queued ahead
         self.n_steps = 0
         self.last_portions: List[int] = []      # tokens of each request in the last step (1: a decoded token)
         self.prompt_tokens = 0          # counters in place of the reference's Prometheus ones
@@ -110,23 +123,55 @@ class Engine:
 
     # -- one step --------------------------------------------------------------------------------
     def step(self) -> int:
-        """Plan and run one step. Returns the number of tokens it ran (0: nothing to do)."""
-        plan = self.scheduler.plan()
-        if not plan:
-            return 0
+        """Plan and run one step, and take its tokens. Returns the number of tokens it ran
+        (0: nothing to do).
+
+        With ``lookahead``, the step after this one is queued before this one's tokens are
+        awaited, where the scheduler knows it without them (``Scheduler.repeats``): the
+        device takes the tokens from the sampler's output, so it goes from one decode step
+        into the next without waiting for the host to read, record, plan and launch. Each
+        call still returns with exactly one more step's tokens recorded. A request that stops
+        at a stop token has then one place in the step that was queued ahead; that place's
+        token is dropped, and its key and value lie beyond the request's end in pages that
+        are freed with it."""
+        flight = self._flight
+        self._flight = None
+        if flight is not None and not any(self._live(p.request) for p in flight.plan):
+            flight = None                 # everyone in it was cancelled or retired meanwhile
+        if flight is None:
+            plan = self.scheduler.plan()
+            if not plan:
+                return 0
+            flight = self._launch(plan, None)
+        if self.lookahead and self.runner.feeds(len(flight.plan)) and self.scheduler.repeats(flight.plan):
+            ahead = [Planned(p.request, [0], True) for p in flight.plan]
+            self._flight = self._launch(ahead, flight.drawn.tokens)
+            self.n_ahead += 1
+        tokens = self.sampler.collect(flight.drawn)
+        for p, token in zip(flight.wanted, tokens):
+            if self._live(p.request):
+                self.record(p.request, token)
+        self.last_portions = [len(p.tokens) for p in flight.plan]
+        self.n_steps += 1
+        return sum(self.last_portions)
+
+    @staticmethod
+    def _live(req: Request) -> bool:
+        return req.row >= 0 and not req.done and not req.cancelled
+
+    def _launch(self, plan, fed) -> "_Flight":
+        """Queue the step of ``plan`` and the choice of its tokens; ``fed``: the tokens of a
+        step planned ahead, on the device."""
         entries = [StepEntry(p.request.row, p.tokens, [len(p.tokens) - 1] if p.wants_logits else [])
                    for p in plan]
-        self.last_portions = [len(p.tokens) for p in plan]
-        logits = self.runner.step(entries, borrow=True)
+        logits = self.runner.step(entries, borrow=True) if fed is None else \
+            self.runner.step(entries, borrow=True, fed=fed)
         wanted = [p for p in plan if p.wants_logits]
-        tokens = self.sampler.sample(logits, [p.request.row for p in wanted])
+        drawn = self.sampler.launch(logits, [p.request.row for p in wanted])
         for p in plan:
-            if not p.request.output:
+            if not p.request.output and fed is None:
                 self.prompt_tokens += len(p.tokens)
-        for p, token in zip(wanted, tokens):
-            self.record(p.request, token)
-        self.n_steps += 1
-        return sum(len(p.tokens) for p in plan)
+        return _Flight(plan, wanted, drawn)
 
     def record(self, req: Request, token: int) -> None:
         """A stop token ends the request and is not kept (model/inference_paged.py:200-211);

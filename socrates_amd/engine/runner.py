@@ -52,16 +52,20 @@ class ModelRunner:
         return runner
 
     @torch.no_grad()
-    def step(self, entries: List[StepEntry], borrow: bool = False) -> torch.Tensor:
+    def step(self, entries: List[StepEntry], borrow: bool = False, fed: torch.Tensor = None) -> torch.Tensor:
         """Returns float32 logits [wanted places, vocab], in the order of the entries and of
         each entry's ``want``. Raises OutOfBlocks if the pages do not suffice (lengths
         are then unchanged; pages already taken stay with their rows). ``borrow``: the
         caller uses the logits before the next step, so a captured step may hand out its own
-        output buffer instead of a copy."""
+        output buffer instead of a copy. ``fed``: int32 [entries] on the device, the one token
+        of each entry where the host does not know it yet (the entries' own tokens are then
+        placeholders); only where ``feeds`` says so."""
         cache = self.cache
         if (self._graphs is not None and len(entries) <= self._graph_max
                 and all(len(e.tokens) == 1 for e in entries)):
-            return self._step_captured(entries, borrow)
+            return self._step_captured(entries, borrow, fed)
+        if fed is not None:
+            raise ValueError("tokens can be fed from the device only to a step that `feeds` admits")
         starts = [cache.length(e.row) for e in entries]
         ctx = build_context(entries, starts, self.ops.device, self.vocab_size, self._upload)
         for e, start in zip(entries, starts):
@@ -95,6 +99,12 @@ class ModelRunner:
         self._graphs = {}
         self._graph_max = max_width
         self._graph_pool = torch.cuda.graph_pool_handle()
+
+    def feeds(self, n_entries: int) -> bool:
+        """Whether a step of ``n_entries`` single tokens can take them from the device
+        (``step(..., fed=)``): such steps are the ones replayed from graphs, whose inputs
+        live at fixed addresses."""
+        return self._graphs is not None and n_entries <= self._graph_max
 
     def _bucket(self, n: int) -> int:
         for b in self._BUCKETS:
@@ -159,12 +169,14 @@ class ModelRunner:
         # through ctx) has to live as long as the graph, so ctx is kept beside it.
         return graph, inputs, staging, logits, ctx
 
-    def _step_captured(self, entries: List[StepEntry], borrow: bool) -> torch.Tensor:
+    def _step_captured(self, entries: List[StepEntry], borrow: bool, fed: torch.Tensor = None) -> torch.Tensor:
         cache = self.cache
         n = len(entries)
         rows = [e.row for e in entries]
         if len(set(rows)) != n:
             raise ValueError("a cache row appears twice in one step")
+        if fed is not None and (fed.dtype != torch.int32 or fed.shape != (n,) or fed.device.type != self.ops.device.type):
+            raise ValueError(f"fed tokens must be int32 [{n}] on {self.ops.device}")
         width = self._bucket(n)
         # key splits of the attention kernel are planned per context bucket, so that a short
         # context is not cut into the many splits a long one needs
@@ -189,6 +201,8 @@ class ModelRunner:
             host[0, i], host[1, i], host[2, i], host[3, i] = token, start, e.row, start + 1
         cache.sync()
         inputs.copy_(staging, non_blocking=True)
+        if fed is not None:
+            inputs[0, :n].copy_(fed)
         copied = copied or torch.cuda.Event()
         copied.record()
         self._staging_read[key] = copied

@@ -189,6 +189,29 @@ class Scheduler:
             budget -= n
         return plan
 
+    def repeats(self, plan: List[Planned]) -> bool:
+        """Whether the step after ``plan`` is known before ``plan``'s tokens are: every
+        running request gets a token from ``plan`` and none reaches its limit with it, nobody
+        is cancelled, nobody who waits could be given a row, and the pages for one more token
+        each are free, so that the next step is one token for each of the same requests
+        whatever the tokens turn out to be (a stop token aside: its request's place in that
+        next step is then wasted, and whoever waits for its row gets it a step later).
+        Changes nothing."""
+        if len(plan) != len(self.running):
+            return False
+        if self.pending and len(self.running) < self.max_batch and self.cache.n_free_rows > 0:
+            return False
+        free = self.cache.free_pages()
+        for p, req in zip(plan, self.running):
+            if (p.request is not req or not p.wants_logits or req.cancelled or req.done
+                    or len(req.output) + 1 >= req.max_new_tokens):
+                return False
+            need = self.cache.pages_needed(req.row, self._cached(req) + 1)
+            if not self._fits(need, free):
+                return False
+            free = [f - max(t, 0) for f, t in zip(free, need)]
+        return True
+
     # -- finishing ---------------------------------------------------------------------------
     def retire_finished(self) -> List[Request]:
         """Close the rows of requests that are done or cancelled; their pages are free

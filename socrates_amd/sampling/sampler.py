@@ -33,19 +33,33 @@ class SamplingParams:
             raise ValueError("temperature must not be negative")
 
 
+@dataclass
+class Drawn:
+    """The tokens of one call of ``Sampler.launch``: on the device at once (``tokens``, int32
+    [n]), on the host once ``ready`` has passed."""
+    tokens: torch.Tensor
+    host: torch.Tensor
+    ready: object = None
+
+
 class Sampler:
     def __init__(self, ops, scalars, upload=None):
         """ops: the kernel set; scalars: the cache manager's RowScalars; upload: int32 numpy
         array -> device tensor (the step function's pinned staging), default a plain copy."""
         self.ops, self.scalars, self.upload = ops, scalars, upload
+        # pinned buffers that the tokens come back through: one more than the calls whose
+        # tokens can be outstanding at a time (a step and the one launched ahead of it)
+        self._ring = [None, None, None]
+        self._turn = 0
 
-    def sample(self, logits: torch.Tensor, rows: Sequence[int]):
-        """One token for each row of ``logits`` (float32 [n, vocab]); ``rows[i]`` is the cache
-        row whose sampling state applies. Returns a list of ints and counts the draws."""
+    def launch(self, logits: torch.Tensor, rows: Sequence[int]) -> Optional[Drawn]:
+        """Queue the choice of one token for each row of ``logits`` (float32 [n, vocab]) and
+        count the draws; ``rows[i]`` is the cache row whose sampling state applies. Does not
+        wait for the device: ``collect`` does. None if there are no rows."""
         if len(rows) != logits.shape[0]:
             raise ValueError("one cache row per row of logits")
         if not len(rows):
-            return []
+            return None
         idx = np.asarray(rows, dtype=np.int64)
         temperature = self.scalars.temperature[idx]
         if not temperature.any():
@@ -63,4 +77,28 @@ class Sampler:
             tokens = self.ops.sample(logits, dev[4 * n:].view(torch.float32),
                                      dev[:2 * n].view(torch.int64), dev[2 * n:4 * n].view(torch.int64))
         self.scalars.draws[idx] += 1
-        return [int(t) for t in tokens.tolist()]
+        if tokens.device.type != "cuda":
+            return Drawn(tokens, tokens)
+        n = tokens.numel()
+        self._turn = (self._turn + 1) % len(self._ring)
+        slot = self._ring[self._turn]
+        if slot is None or slot[0].numel() < n:
+            slot = self._ring[self._turn] = (torch.empty(max(64, n), dtype=torch.int32).pin_memory(),
+                                             torch.cuda.Event())
+        host, ready = slot[0][:n], slot[1]
+        host.copy_(tokens, non_blocking=True)
+        ready.record()
+        return Drawn(tokens, host, ready)
+
+    @staticmethod
+    def collect(drawn: Optional[Drawn]):
+        """The tokens of a ``launch`` as a list of ints, once the device has them."""
+        if drawn is None:
+            return []
+        if drawn.ready is not None:
+            drawn.ready.synchronize()
+        return [int(t) for t in drawn.host.tolist()]
+
+    def sample(self, logits: torch.Tensor, rows: Sequence[int]):
+        """``launch`` and ``collect`` in one: a list of ints, one token per row."""
+        return self.collect(self.launch(logits, rows))

@@ -155,6 +155,62 @@ def test_command_line_with_a_preset(tmp_path):
     assert shown == [" ".join(map(str, want))]
 
 
+def test_steps_queued_ahead_change_no_token(tmp_path):
+    """The engine queues the next decode step before it has read the last one's tokens.
+    Requests that stop at a stop token in the middle (the step queued ahead then has a
+    wasted place), limits of different lengths, a request submitted while a step is ahead,
+    a cancelled one, temperature, and a pool in which the step ahead does not always find
+    its pages: the tokens are those of an engine that never queues ahead, and in float32
+    the plain run's."""
+    from socrates_amd.engine import Engine
+    from socrates_amd.sampling import SamplingParams
+    folder = write_tiny(tmp_path / "A", TINY_A, seed=2)
+    cfg, w = plain.read_folder(folder, torch.float64)
+    prompts = random_prompts([5, 17, 33, 2, 21], cfg["vocab_size"], seed=3)
+    free = [plain.greedy(cfg, w, p, 20) for p in prompts]
+    # request i stops at the token that the plain run has at place stops[i] (if it does not
+    # appear earlier, which the expected output below accounts for)
+    stops, limits = [6, 11, None, 3, None], [20, 20, 9, 20, 14]
+    want, eos = [], []
+    for out, stop, limit in zip(free, stops, limits):
+        eos.append(() if stop is None else (out[stop],))
+        cut = out.index(out[stop]) if stop is not None else len(out)
+        want.append(out[:min(cut, limit)])
+
+    def run(lookahead, num_blocks=None):
+        engine = Engine(str(folder), dtype=torch.float32, max_batch=4, max_len=64, max_new_tokens=20,
+                        block_size=16, num_blocks=num_blocks, lookahead=lookahead)
+        reqs = [engine.submit(p, sampling=SamplingParams(max_new_tokens=n, eos_token_ids=e))
+                for p, n, e in list(zip(prompts, limits, eos))[:4]]
+        for _ in range(4):
+            engine.step()
+        reqs.append(engine.submit(prompts[4], sampling=SamplingParams(max_new_tokens=limits[4], eos_token_ids=eos[4])))
+        doomed = engine.submit(prompts[0], sampling=SamplingParams(max_new_tokens=20, eos_token_ids=()))
+        while not doomed.output:
+            engine.step()
+        doomed.cancelled = True
+        engine.run()
+        engine.cache.check()
+        assert not engine.cache.open_rows and engine.cache.n_free_pages == (num_blocks or 16)
+        return [r.output for r in reqs], engine
+
+    got, engine = run(True)
+    assert got == want
+    assert engine.n_ahead >= 8, engine.n_ahead
+    plainly, engine = run(False)
+    assert plainly == want and engine.n_ahead == 0
+    tight, engine = run(True, num_blocks=7)
+    assert tight == want
+
+    outs = []
+    for lookahead in (True, False):
+        engine = Engine(str(folder), dtype=torch.bfloat16, max_batch=4, max_len=64, max_new_tokens=16,
+                        block_size=16, lookahead=lookahead)
+        outs.append(engine.generate(prompts, temperature=0.7, seed=11, eos_token_ids=()))
+        assert (engine.n_ahead > 0) == lookahead
+    assert outs[0] == outs[1]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_engine_under_page_pressure(tmp_path, dtype):
     """Pools so small that requests wait, have their portions shortened and are preempted,
