@@ -122,6 +122,61 @@ def test_preempts_the_youngest_when_a_running_request_needs_a_page():
     assert len(young.output) == 8 and cache.n_free_pages == 4 and s.n_preemptions == 1
 
 
+def test_when_the_next_step_is_known_before_the_tokens():
+    """``repeats``, asked as the engine asks it (the plan's step is queued, its tokens are not
+    there yet): the step after a plan is one token for each of the same requests, whatever
+    the plan's tokens are, only if every running request is in the plan and gets a token
+    from it, none reaches its limit with that token, nobody who waits could be given a row,
+    nobody is cancelled and the pages for one more token each are free. It changes nothing."""
+    def queue(cache, plan):
+        for p in plan:
+            start = cache.length(p.request.row)
+            cache.reserve(p.request.row, start + len(p.tokens))
+            cache.advance(p.request.row, len(p.tokens))
+
+    def tokens(plan, token=7):
+        for p in plan:
+            if p.wants_logits:
+                p.request.output.append(token)
+                p.request.done = len(p.request.output) >= p.request.max_new_tokens
+
+    s, cache = sched(rows=2, pages=8, budget=16, bs=8)
+    a, b = req(5, max_new=3), req(20, max_new=6)
+    s.submit(a), s.submit(b)
+    plan = s.plan()                             # a whole, 11 tokens of b: b gets no token yet
+    queue(cache, plan)
+    assert not s.repeats(plan)
+    tokens(plan)
+    plan = s.plan()                             # a decodes, b's last 9 tokens: both get a token
+    queue(cache, plan)
+    free = cache.free_pages()
+    assert s.repeats(plan) and cache.free_pages() == free and len(s.running) == 2
+    c = req(3)
+    s.submit(c)                                 # both rows are taken: c cannot be admitted anyway
+    assert s.repeats(plan)
+    a.cancelled = True
+    assert not s.repeats(plan)
+    a.cancelled = False
+    tokens(plan)                                # a has 2 of 3
+    plan = s.plan()
+    queue(cache, plan)
+    assert len(a.output) == 2 and not s.repeats(plan)       # this step's token is a's last
+    tokens(plan)
+    assert a.done
+    plan = s.plan()                             # a retired, c admitted beside b
+    queue(cache, plan)
+    assert [p.request for p in plan] == [b, c] and s.repeats(plan)
+    # pages: two requests that fill the pool's two pages; the next token of the first needs a third
+    s, cache = sched(rows=2, pages=2, budget=16, bs=8, max_len=16)
+    a, b = req(8, max_new=8), req(7, max_new=8)
+    s.submit(a), s.submit(b)
+    plan = s.plan()
+    assert [len(p.tokens) for p in plan] == [8, 7]
+    queue(cache, plan)
+    assert not s.repeats(plan)
+    cache.check()
+
+
 def test_cancelled_requests_are_dropped_and_freed():
     s, cache = sched(pages=8)
     a, b, c = req(9), req(9), req(9)
