@@ -206,6 +206,8 @@ def main(argv=None):
     ap.add_argument("--split-keys", type=int, default=None, help="key splits of the decode attention: fewest keys of a split")
     ap.add_argument("--no-fused-norms", action="store_true",
                     help="decode steps with the residual sums and norms in kernels of their own")
+    ap.add_argument("--sweep-rows", type=int, default=None,
+                    help="rows of a decode step from which its products take the sweep form (0: never)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is "
@@ -230,6 +232,8 @@ def main(argv=None):
     config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
     V = config.vocab_size
     engine.runner.ops.fuse_norms = not args.no_fused_norms
+    if args.sweep_rows is not None:
+        engine.runner.ops.sweep_rows = args.sweep_rows
     if args.split_waves:
         engine.runner.ops.split_target_waves = args.split_waves
     if args.split_keys:

@@ -655,3 +655,197 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
     SOC_SK(bf16, 4, 2);
 #undef SOC_SK
 }
+
+// ---------------------------------------------------------------------------------------------
+// Sweep form of the skinny product (M <= 16; plain, SCALED and SWIGLU forms, K not split over
+// workgroups). In the kernel above every workgroup reads all rows of x for its 16 weight
+// rows, and with some hundred workgroups per product that re-reading costs a quarter of the
+// kernel's time at 8 rows and a third at 16 (a build without the loads of x runs at the
+// one-row speed whatever M is). Here a product has at most one workgroup per compute unit,
+// of 16 waves that split K as before; a wave keeps its slices of x in registers for the
+// whole kernel (at most 8 steps of 32 k, so K up to 4,096), and the workgroup sweeps over
+// weight tiles g, g + G, g + 2 G, ...: per tile a wave loads only weights, multiplies, and
+// leaves its sums in LDS, where the first four waves add them and do the epilogue while the
+// others go on. The weights of two tiles are on their way at any time, and x is read once per
+// workgroup. At one row the form of a workgroup per tile streams the weights 8 % faster; from
+// 4 rows on this one wins (gate+up of a 4B-sized layer at 8 rows: 23.3 against 27.0 us, at 16
+// rows 24.8 against 33.8 us; the output head of 151,936 rows at 8 rows: 141 against 169 us).
+// SWIGLU: an item is a pair of tiles (gate rows, then up rows of the same 16 outputs), swept
+// one after the other; the gate sums wait in registers for the up sums.
+// (The form with a residual epilogue stays with the kernel above: its few tiles with a long K
+// need K split over workgroups, and workgroups that sweep and meet in memory were measured
+// at twice its time.)
+constexpr uint32_t SW_NOWHERE = 0xfffffff0u;        // an offset past the end of every buffer: reads as zeros, asks memory for nothing
+
+struct SwPlan {
+    int k_per_wave;                 // a multiple of 32
+    int items;                      // weight tiles (tile pairs with SWIGLU)
+};
+
+template <typename TC, int MODE, int MAXS>
+__global__ void __launch_bounds__(1024)
+gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C, int M,
+                       int N, int K, SwPlan pl, SkNorm nm) {
+    constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED;
+    static_assert(!(MODE & SK_ADDNORM), "the residual epilogue stays with the skinny kernel");
+    constexpr int SUB = SWIGLU ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) float red[2][16 * 256];     // [tile parity][wave][lane][4]
+    __shared__ float row_fac[16];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
+    const int n_waves = blockDim.x / SOC_WAVE;
+    const int g = blockIdx.x, G = gridDim.x;
+    const int li = lane % 16, lk = (lane / 16) * 8;
+    const int k_begin = wave * pl.k_per_wave, k_end = min(K, k_begin + pl.k_per_wave);
+    const int my_items = pl.items > g ? (pl.items - g + G - 1) / G : 0;
+    const int n_sub = my_items * SUB;                                    // tiles this workgroup sweeps
+    auto tile_of = [&](int q) {
+        const int item = g + (q / SUB) * G;
+        return SWIGLU ? 2 * item + (q % SUB) : item;
+    };
+
+    // Both operands through buffer descriptors that end with their matrices: rows of x beyond
+    // M, weight rows beyond N and every slice chosen to lie nowhere read as zeros. No branch
+    // lies between a load and its use.
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, M * K * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(W), (short)0, (int)((size_t)N * K * 2), 0x00020000);
+    uint4 xr[MAXS];
+    uint32_t k_off[MAXS];                               // byte offset of the slice in its row, or nowhere
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) {
+        const int k = k_begin + 32 * s + lk;
+        k_off[s] = k < k_end ? (uint32_t)(k * 2) : SW_NOWHERE;
+        xr[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                    x_rsrc, k < k_end ? (uint32_t)((li * K + k) * 2) : SW_NOWHERE, 0, 0));
+    }
+    auto load_w = [&](uint4 (&wb)[MAXS], int q) {
+        const bool live = q < n_sub;                    // the same for the whole workgroup
+        const uint32_t row = live ? (uint32_t)((size_t)(tile_of(live ? q : 0) * 16 + li) * K * 2) : 0u;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s)
+            wb[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                        w_rsrc, live && k_off[s] != SW_NOWHERE ? row + k_off[s] : SW_NOWHERE, 0, 0));
+    };
+    auto compute = [&](const uint4 (&wb)[MAXS]) {
+        f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wb[s]),
+                                                          __builtin_bit_cast(bf16x8, xr[s]), acc, 0, 0, 0);
+        return acc;
+    };
+
+    uint4 wa[MAXS], wb2[MAXS];
+    load_w(wa, 0);
+    load_w(wb2, 1);
+    if constexpr (SCALED) {
+        // the norm's factor of every row, once per workgroup, while the first loads are on their way
+        const int stride = sk_ssq_stride(nm.ssq_tiles);
+        for (int m = wave; m < 16; m += n_waves) {
+            float s = 0.f;
+            if (m < M)
+                for (int t = lane; t < nm.ssq_tiles; t += SOC_WAVE) s += nm.ssq_in[(size_t)m * stride + t];
+            s = wave_sum(s);
+            if (lane == 0) row_fac[m] = 1.0f / sqrtf(s * nm.inv_dim + nm.eps);
+        }
+    }
+
+    // A reducer (the first 256 threads): row rm of x, column rc of the tile. acc[e] of lane l of
+    // a wave is the partial sum for row l % 16 and column 4 (l / 16) + e.
+    const int rm = (tid % 256) / 16, rc = tid % 16;
+    const int red_at = ((rc / 4) * 16 + rm) * 4 + rc % 4;
+    float held = 0.f;                                   // SWIGLU: the gate sum, until the up sum is there
+    auto leave = [&](f32x4 acc, int p) {
+        *reinterpret_cast<float4*>(&red[p][wave * 256 + lane * 4]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        __syncthreads();
+    };
+    auto finish = [&](int q, int p) {
+        if (tid >= 256 || q >= n_sub) return;           // whole waves leave
+        const int tile = tile_of(q);
+        float sum = 0.f;
+        for (int w = 0; w < n_waves; ++w) sum += red[p][w * 256 + red_at];
+        if constexpr (SCALED) sum *= row_fac[rm];
+        if constexpr (SWIGLU) {
+            if (q % 2 == 0) { held = sum; return; }
+            const int col = (tile / 2) * 16 + rc, half = N / 2;
+            if (rm < M && col < half) C[(size_t)rm * half + col] = from_float<TC>(sum * (held / (1.0f + expf(-held))));
+        } else {
+            const int n = tile * 16 + rc;
+            if (rm < M && n < N) C[(size_t)rm * N + n] = from_float<TC>(sum);
+        }
+    };
+
+    // Two tiles' weights are on their way: a buffer is asked for anew as soon as its tile's
+    // sums are in LDS, before the epilogue. The sums of a tile go to the half of `red` of its
+    // parity: the reducers read one half while the next tile's sums are written to the other,
+    // and one barrier per tile orders both. Past the end of the sweep a round loads zeros
+    // from nowhere and has no epilogue, but the barrier all the same.
+    for (int q = 0; q < n_sub; q += 2) {
+        leave(compute(wa), 0);
+        load_w(wa, q + 2);
+        finish(q, 0);
+        leave(compute(wb2), 1);
+        load_w(wb2, q + 3);
+        finish(q + 1, 1);
+    }
+}
+
+// Shape of a sweep for an [M <= 16] x [N, K] product: waves per workgroup and workgroups; 0
+// if the sweep form does not apply (K longer than 16 waves x 256). The tiles (pairs) are
+// shared out so that the GPU's 256 compute units get at most one workgroup each, with equal
+// numbers of tiles as far as that goes.
+SOC_EXPORT int soc_gemm_sweep_plan(int N, int K, int swiglu, int* n_waves, int* workgroups) {
+    const int nw = 16;
+    if (K > nw * 256) return 0;
+    const int items = swiglu ? N / 32 : (N + 15) / 16;
+    if (items < 1) return 0;
+    const int per_wg = (items + 255) / 256;
+    *n_waves = nw;
+    *workgroups = (items + per_wg - 1) / per_wg;
+    return 1;
+}
+
+// mode: SK_SWIGLU (C [M, N / 2], N a multiple of 32) or 0 (C [M, N] in c_dtype), each with or
+// without SK_SCALED (ssq_in, ssq_tiles, norm_dim, eps; bfloat16 output). K / n_waves rounded
+// up to 32 must not exceed 256. The matrices lie below 4 GiB.
+SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
+                                   int mode, int n_waves, int workgroups, const float* ssq_in, int ssq_tiles,
+                                   int norm_dim, float eps, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 || K < 8 || !C) return (int)hipErrorInvalidValue;
+    if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;
+    if (n_waves < 1 || n_waves > 16 || workgroups < 1) return (int)hipErrorInvalidValue;
+    const bool swiglu = mode & SK_SWIGLU, scaled = mode & SK_SCALED;
+    if ((mode & ~3) || (swiglu && N % 32)) return (int)hipErrorInvalidValue;
+    if (scaled && (!ssq_in || ssq_tiles < 1 || norm_dim < 1)) return (int)hipErrorInvalidValue;
+    if (c_dtype != 0 && c_dtype != 1) return (int)hipErrorInvalidValue;
+    if (c_dtype == 0 && mode != 0) return (int)hipErrorInvalidValue;            // float32 output: the plain form only
+    SwPlan pl;
+    pl.k_per_wave = ((K + n_waves - 1) / n_waves + 31) / 32 * 32;
+    if (pl.k_per_wave > 256) return (int)hipErrorInvalidValue;
+    pl.items = swiglu ? N / 32 : (N + 15) / 16;
+    SkNorm nm{};
+    nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
+    const dim3 grid(workgroups < pl.items ? workgroups : pl.items), block(n_waves * 64);
+    const int steps = pl.k_per_wave / 32;
+#define SOC_SW(TC_, MODE_, MAXS_) \
+    hipLaunchKernelGGL((gemm_bf16_sweep_kernel<TC_, MODE_, MAXS_>), grid, block, 0, stream, (const bf16*)X, \
+                       (const bf16*)W, (TC_*)C, M, N, K, pl, nm)
+#define SOC_SW_STEPS(TC_, MODE_)                                                           \
+    do {                                                                                   \
+        if (steps <= 2) SOC_SW(TC_, MODE_, 2); else if (steps <= 4) SOC_SW(TC_, MODE_, 4); \
+        else if (steps <= 5) SOC_SW(TC_, MODE_, 5); else SOC_SW(TC_, MODE_, 8);            \
+    } while (0)
+    if (c_dtype == 0) { SOC_SW_STEPS(float, 0); return soc_last_error(); }
+    switch (mode) {
+        case 0: SOC_SW_STEPS(bf16, 0); break;
+        case SK_SCALED: SOC_SW_STEPS(bf16, SK_SCALED); break;
+        case SK_SWIGLU: SOC_SW_STEPS(bf16, SK_SWIGLU); break;
+        case SK_SWIGLU | SK_SCALED: SOC_SW_STEPS(bf16, SK_SWIGLU | SK_SCALED); break;
+        default: return (int)hipErrorInvalidValue;
+    }
+#undef SOC_SW_STEPS
+#undef SOC_SW
+    return soc_last_error();
+}

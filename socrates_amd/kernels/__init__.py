@@ -54,6 +54,8 @@ _GEMM_SIGNATURES = {
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
     "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P, I, I, F, P],
     "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, I, P, P, P],
+    "soc_gemm_bf16_sweep": [P, P, P, I, I, I, I, I, I, I, P, I, I, F, P],
+    "soc_gemm_sweep_plan": [I, I, I, P, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -68,7 +70,7 @@ _ATTENTION_SIGNATURES = {
 def _declare(lib, signatures):
     for name, argtypes in signatures.items():
         fn = getattr(lib, name)
-        fn.argtypes, fn.restype = argtypes, (None if name.endswith("_plan") else c_int)
+        fn.argtypes, fn.restype = argtypes, (None if name == "soc_gemm_skinny_plan" else c_int)
 
 
 MAX_KEY_SPLITS = 256    # of the MFMA attention: 64 workgroups of four splits meet per task
@@ -147,6 +149,13 @@ class HipKernels:
         # package's tiled MFMA kernel
         self.library_gemm = True
         self.swiglu_waves = 8           # waves of the fused gate+up product (measured: 4, 8, 16 within 5 %)
+        # The sweep form of the skinny product (one workgroup per compute unit keeps its slices
+        # of x in registers and walks over the weight tiles): from this many rows of x on, for
+        # products of at least ``sweep_min_items`` weight tiles (pairs of them with SwiGLU).
+        # Measured on an MI355X at 4B-sized layers: at one row it streams the weights 8 % slower
+        # than a workgroup per tile, from 4 rows on it wins, by a quarter at 16 rows.
+        self.sweep_rows = 4             # 0: never
+        self.sweep_min_items = 256
         # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
         self.fuse_norms = True
@@ -264,6 +273,10 @@ class HipKernels:
             self._want(x, "x")
             self._want(w_gate_up, "weight", None, (N, K))
             out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
+            plan = self._sweep_plan(M, N, K, swiglu=True)
+            if plan is not None:
+                self._sweep(plan, x, w_gate_up, out, self._SK_SWIGLU, self._owed_args(owed, M, K), what="linear_swiglu")
+                return out
             n_waves = self.swiglu_waves          # half of them per tile (gate, up), splitting K
             while n_waves > 2 and K // (n_waves // 2) < 128:
                 n_waves //= 2
@@ -274,6 +287,31 @@ class HipKernels:
                                                           self._stream()), "linear_swiglu")
             return out
         return self.swiglu(self.linear(owed if owed is not None else x, w_gate_up), interleave)
+
+    _SK_SWIGLU, _SK_SCALED = 1, 2
+
+    def _sweep_plan(self, M, N, K, swiglu=False):
+        """(waves, workgroups) if this product of at most 16 rows takes the sweep form."""
+        if not self.sweep_rows or M < self.sweep_rows or M > 16 or K % 8 or K < 8:
+            return None
+        nw, wgs = c_int(0), c_int(0)
+        if not self._gemm.soc_gemm_sweep_plan(c_int(N), c_int(K), c_int(1 if swiglu else 0), ctypes.byref(nw),
+                                              ctypes.byref(wgs)):
+            return None
+        items = N // 32 if swiglu else (N + 15) // 16
+        if items < self.sweep_min_items or (N + 32) * K * 2 >= 0xfffffff0:
+            return None
+        return nw.value, wgs.value
+
+    def _sweep(self, plan, x, w, out, mode, owed_args=(None, 0, 0, 0.0), what="linear"):
+        (M, K), N = x.shape, w.shape[0]
+        ssq, tiles, dim, eps = owed_args
+        if ssq is not None:
+            mode |= self._SK_SCALED
+        _check(self._gemm.soc_gemm_bf16_sweep(
+            _ptr(x), _ptr(w), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(_DTYPE_CODE[out.dtype]), c_int(mode),
+            c_int(plan[0]), c_int(plan[1]), ssq, c_int(tiles), c_int(dim), c_float(eps), self._stream()),
+            f"{what} (sweep) [{M}x{K}] x [{N}x{K}]^T")
 
     def _owed_args(self, owed, M, K):
         """(ssq pointer, tiles, dim, eps) of a NormOwed input, checked; nulls for a plain one."""
@@ -421,7 +459,14 @@ class HipKernels:
             if choice == "library":
                 out = by_library()
                 return out.unsqueeze(0) if allow_partial else out
+        explicit = row_tiles > 0 or n_waves or k_splits
         row_tiles = max(row_tiles, 0)                     # -1: the skinny kernel, whatever the table says
+        if own and not explicit and not allow_partial:
+            plan = self._sweep_plan(M, N, K)
+            if plan is not None:
+                out = torch.empty((M, N), dtype=out_dtype, device=self.device)
+                self._sweep(plan, x, w, out, 0)
+                return out
         if own:
             if not (row_tiles and n_waves and k_splits):
                 rw, nw, ks = c_int(0), c_int(0), c_int(0)
@@ -466,6 +511,10 @@ class HipKernels:
         if out_dtype != torch.bfloat16 or not 0 < M <= 16 or K % 8:
             raise KernelError("rows owed a norm go to bfloat16 products of at most 16 rows")
         out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
+        plan = self._sweep_plan(M, N, K) if not n_waves else None
+        if plan is not None:
+            self._sweep(plan, x, w, out, 0, self._owed_args(owed, M, K))
+            return out
         if not n_waves:
             n_waves = 8
             while n_waves > 1 and K // n_waves < 128:

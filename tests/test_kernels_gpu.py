@@ -217,6 +217,57 @@ def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
     torch.testing.assert_close(r.double(), want_res, atol=2e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("M,d,K", [(1, 64, 64), (8, 2560, 4096), (16, 72, 200), (5, 104, 4088), (3, 4096, 96),
+                                   (11, 2560, 2568), (7, 330, 1000), (16, 6144, 2560), (4, 48, 8)])
+def test_sweep_form_of_the_skinny_products(kernel_sets, M, d, K):
+    """The products of at most 16 rows in their sweep form (a workgroup keeps its slices of x
+    in registers and walks over the weight tiles), forced on at every size: plain, with
+    float32 output, and the two kinds of product that consume rows owed a norm (plain and
+    gate / up with the activation), against float64 and against the form of a workgroup per
+    tile. Rows are scaled very differently, so a factor applied to the wrong row shows. K
+    beyond what a workgroup's waves hold stays with the other form."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    y, w = rnd((M, K), torch.bfloat16, 50), rnd((d, K), torch.bfloat16, 51, K ** -0.5)
+    res = rnd((M, d), torch.float32, 52) * torch.logspace(-2, 2, M, device=DEV)[:, None]
+    gain = (1 + 0.3 * torch.randn(d)).to(DEV)
+    kept = (hip.sweep_rows, hip.sweep_min_items)
+    assert hip._sweep_plan(16, 2560, 9728) is None and hip._sweep_plan(17, 2560, 2560) is None
+    assert hip._sweep_plan(8, 19456, 2560, swiglu=True) == (16, 203)
+
+    def run(sweep):
+        hip.sweep_rows, hip.sweep_min_items = (1, 1) if sweep else (0, 1)
+        assert (hip._sweep_plan(M, d, K) is not None) == sweep
+        out = {"plain": hip.linear(y, w), "f32": hip.linear(y, w, out_dtype=torch.float32)}
+        r = res.clone()
+        owed = hip.linear_add_norm(y, w, r, gain, 1e-6)
+        if d % 8 == 0:
+            N2 = 331 if d < 1000 else 6144
+            w2 = rnd((N2, d), torch.bfloat16, 53, d ** -0.5)
+            out["owed_plain"] = hip.linear(owed, w2)
+            ff = 160 if d < 1000 else 9728
+            wgu = rnd((2 * ff, d), torch.bfloat16, 54, d ** -0.5)
+            out["owed_swiglu"] = hip.linear_swiglu(owed, wgu, 16)
+            out["swiglu"] = hip.linear_swiglu(owed.x, wgu, 16)
+        return out, r
+
+    try:
+        got, r = run(True)
+        want, _ = run(False)
+    finally:
+        hip.sweep_rows, hip.sweep_min_items = kept
+    exact = y.double() @ w.double().T
+    torch.testing.assert_close(got["f32"].double(), exact, atol=3e-5 * max(1, K / 512) ** 0.5, rtol=3e-5)
+    close(got["plain"], exact, torch.bfloat16)
+    if d % 8 == 0:
+        normed = r.double() * torch.rsqrt((r.double() ** 2).mean(-1, keepdim=True) + 1e-6) * gain.double()
+        N2 = 331 if d < 1000 else 6144
+        close(got["owed_plain"], normed @ rnd((N2, d), torch.bfloat16, 53, d ** -0.5).double().T, torch.bfloat16)
+    for name in got:
+        # the two forms add K in another order: equal to a rounding of the output type
+        tol = dict(atol=1e-4, rtol=1e-4) if got[name].dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(got[name].float(), want[name].float(), **tol)
+
+
 def test_linear_float32_is_not_reduced_precision(kernel_sets):
     """Values that bfloat16 or a 19-bit matrix mode would round away survive."""
     hip, _ = kernel_sets[torch.float32]
