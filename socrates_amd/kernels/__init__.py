@@ -153,8 +153,9 @@ class HipKernels:
         # of x in registers and walks over the weight tiles): from this many rows of x on, for
         # products of at least ``sweep_min_items`` weight tiles (pairs of them with SwiGLU).
         # Measured on an MI355X at 4B-sized layers: at one row it streams the weights 8 % slower
-        # than a workgroup per tile, from 4 rows on it wins, by a quarter at 16 rows.
-        self.sweep_rows = 4             # 0: never
+        # than a workgroup per tile, at two rows a decode step takes the same time either way,
+        # from three rows on it wins, by a quarter at 16 rows.
+        self.sweep_rows = 3             # 0: never
         self.sweep_min_items = 256
         # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
