@@ -314,7 +314,7 @@ template <typename TC, int MT, int RW, int MODE = 0>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, RW, MODE))
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
-                        int k_per_wave, SkNorm nm) {
+                        int k_per_wave, SkNorm nm, int w_tiled = 0) {
     constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED, ADDNORM = MODE & SK_ADDNORM;
     static_assert(!(SCALED || ADDNORM) || (MT == 1 && RW == 1), "the norm forms take one tile of each");
     __shared__ float red[sk_max_waves(MT, RW, MODE) * MT * RW * 256];
@@ -331,6 +331,11 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     const int split_end = min(K, split_begin + k_per_split);
     const int k_begin = split_begin + (wave % k_waves) * k_per_wave;
     const int k_end = min(split_end, k_begin + k_per_wave);
+    // The weights lie row by row, [N, K], or by tile (w_tiled: [N / 16, K / 32, 16, 32], N a
+    // multiple of 16 and K of 32): a wave's load of 16 rows x 32 k is then 1 KB in one piece
+    // instead of sixteen pieces of 64 bytes. Either way a tile of 16 rows starts at 16 K t.
+    const int w_rs = w_tiled ? 32 : K;              // elements from a row of a tile to the next
+    const int w_ss = w_tiled ? 512 : 32;            // elements from a step of 32 k to the next
     // Element offsets of this lane's rows (offsets, not pointers: the loads stay global
     // loads); a row outside the matrix is never loaded.
     size_t w_off[RW];
@@ -338,7 +343,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
         w_ok[r] = n0 + r * 16 + li < N;
-        w_off[r] = (size_t)(w_ok[r] ? n0 + r * 16 + li : 0) * K + lk;
+        w_off[r] = w_ok[r] ? (size_t)(n0 + r * 16) * K + (size_t)li * w_rs + lk : (size_t)lk;
     }
     // X is read through a buffer descriptor that covers its M rows: a lane whose row lies
     // outside (M = 8 leaves half of the 16 lanes of a tile without one) gets zeros and asks
@@ -372,7 +377,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 #define SK_LOAD(B, K0)                                                                              \
     _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u) {                                          \
         _Pragma("unroll") for (int r = 0; r < RW; ++r)                                               \
-            B.w[r][u] = *reinterpret_cast<const uint4*>(W + w_off[r] + (K0) + 32 * u);               \
+            B.w[r][u] = *reinterpret_cast<const uint4*>(W + w_off[r] + (size_t)((K0) / 32 + u) * w_ss); \
         _Pragma("unroll") for (int t = 0; t < MT; ++t)                                               \
             B.x[t][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(              \
                 x_rsrc, x_off[t] + (uint32_t)(((K0) + 32 * u) * 2), 0, 0));                          \
@@ -416,7 +421,8 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
             const bool in = kk + lk < k_end;
 #pragma unroll
             for (int r = 0; r < RW; ++r)
-                b0.w[r][u] = in ? *reinterpret_cast<const uint4*>(W + w_off[r] + kk) : make_uint4(0u, 0u, 0u, 0u);
+                b0.w[r][u] = in ? *reinterpret_cast<const uint4*>(W + w_off[r] + (size_t)(kk / 32) * w_ss + kk % 32)
+                                : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
             for (int t = 0; t < MT; ++t)
                 b0.x[t][u] = in ? __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
@@ -522,13 +528,13 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 
 template <typename TC, int MT, int RW>
 static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N, int K,
-                         int n_waves, int k_splits, hipStream_t stream) {
+                         int n_waves, int k_splits, int w_tiled, hipStream_t stream) {
     // ranges are multiples of the 128-k step, so only the end of K can be a partial step
     const int k_per_split = ((K + k_splits - 1) / k_splits + SK_STEP - 1) / SK_STEP * SK_STEP;
     const int k_per_wave = ((k_per_split + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT, RW>), dim3((N + 16 * RW - 1) / (16 * RW), k_splits),
                        dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (TC*)C, Cpart, M, N,
-                       K, k_per_split, k_per_wave, SkNorm{});
+                       K, k_per_split, k_per_wave, SkNorm{}, w_tiled);
     return soc_last_error();
 }
 
@@ -539,8 +545,9 @@ static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, in
 // factor is applied to the sums (the SCALED form above). bfloat16 output only then.
 SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C, int M, int N, int K,
                                            int c_dtype, int n_waves, const float* ssq_in, int ssq_tiles,
-                                           int norm_dim, float eps, hipStream_t stream) {
+                                           int norm_dim, float eps, int w_tiled, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23) || N % 32) return (int)hipErrorInvalidValue;
     if (n_waves < 2 || n_waves > SK_MAX_WAVES_SWIGLU || n_waves % 2) return (int)hipErrorInvalidValue;
     if (ssq_in && (ssq_tiles < 1 || ssq_tiles > 16 * SK_SSQ_MAX_PAIRS || norm_dim < 1 || c_dtype != 1))
@@ -553,15 +560,15 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
     if (ssq_in)
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU | SK_SCALED>), dim3(N / 32, 1),
                            dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (bf16*)C,
-                           (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm);
+                           (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, w_tiled);
     else if (c_dtype == 0)
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (float*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave, nm);
+                           k_per_split, k_per_wave, nm, w_tiled);
     else
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave, nm);
+                           k_per_split, k_per_wave, nm, w_tiled);
     return soc_last_error();
 }
 
@@ -578,8 +585,9 @@ SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, 
                                          int n_waves, const float* ssq_in, int ssq_tiles, int norm_dim,
                                          float eps, float* residual, const float* gain, void* x_out,
                                          float* ssq_out, int k_splits, float* split_sums, int* split_count,
-                                         hipStream_t stream) {
+                                         int w_tiled, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > SK_MAX_WAVES_SWIGLU) return (int)hipErrorInvalidValue;
     if (!ssq_in && !residual) return (int)hipErrorInvalidValue;
@@ -597,7 +605,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, 
     const dim3 grid((N + 15) / 16, k_splits), block(n_waves * 64);
 #define SOC_SKN(MODE_) \
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, MODE_>), grid, block, 0, stream, (const bf16*)X, \
-                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm)
+                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, w_tiled)
     if (ssq_in && residual) SOC_SKN(SK_SCALED | SK_ADDNORM);
     else if (residual) SOC_SKN(SK_ADDNORM);
     else SOC_SKN(SK_SCALED);
@@ -627,11 +635,13 @@ SOC_EXPORT void soc_gemm_skinny_plan(int M, int N, int K, int allow_split, int* 
 }
 
 // M <= 64, K a multiple of 8. k_splits == 1: C [M, N] in c_dtype. k_splits > 1: float32
-// partial sums Cpart [k_splits, M, N] (C is not written).
+// partial sums Cpart [k_splits, M, N] (C is not written). w_tiled (here and in the entry
+// points around): W lies by tile, [N / 16, K / 32, 16, 32], N a multiple of 16 and K of 32.
 SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N,
                                     int K, int c_dtype, int row_tiles, int n_waves, int k_splits,
-                                    hipStream_t stream) {
+                                    int w_tiled, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
     if (M > 64 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;   // 32-bit byte offsets into X
     if (n_waves < 1 || n_waves > (M <= 16 && row_tiles == 1 ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES) || k_splits < 1 ||
         k_splits > 65535)
@@ -640,7 +650,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     if (row_tiles != 2 && !((row_tiles == 4 || row_tiles == 1) && MT == 1)) return (int)hipErrorInvalidValue;
 #define SOC_SK(TC_, MT_, RW_) \
-    return launch_skinny<TC_, MT_, RW_>(X, W, C, Cpart, M, N, K, n_waves, k_splits, stream)
+    return launch_skinny<TC_, MT_, RW_>(X, W, C, Cpart, M, N, K, n_waves, k_splits, w_tiled, stream)
     if (c_dtype == 0) {
         if (MT == 1 && row_tiles == 4) SOC_SK(float, 1, 4);
         if (MT == 1 && row_tiles == 1) SOC_SK(float, 1, 1);
@@ -685,7 +695,7 @@ struct SwPlan {
 template <typename TC, int MODE, int MAXS>
 __global__ void __launch_bounds__(1024)
 gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C, int M,
-                       int N, int K, SwPlan pl, SkNorm nm) {
+                       int N, int K, SwPlan pl, SkNorm nm, int w_tiled) {
     constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED;
     static_assert(!(MODE & SK_ADDNORM), "the residual epilogue stays with the skinny kernel");
     constexpr int SUB = SWIGLU ? 2 : 1;
@@ -710,18 +720,21 @@ gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, T
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, M * K * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(W), (short)0, (int)((size_t)N * K * 2), 0x00020000);
+    // (the weights row by row or by tile, as in the skinny kernel)
+    const int w_rs = w_tiled ? 32 : K, w_ss = w_tiled ? 512 : 32;
     uint4 xr[MAXS];
-    uint32_t k_off[MAXS];                               // byte offset of the slice in its row, or nowhere
+    uint32_t k_off[MAXS];                               // byte offset of the slice from its tile's row 0, or nowhere
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = k_begin + 32 * s + lk;
-        k_off[s] = k < k_end ? (uint32_t)(k * 2) : SW_NOWHERE;
+        k_off[s] = k < k_end ? (uint32_t)((((k_begin / 32 + s) * w_ss) + li * w_rs + lk) * 2) : SW_NOWHERE;
         xr[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
                     x_rsrc, k < k_end ? (uint32_t)((li * K + k) * 2) : SW_NOWHERE, 0, 0));
     }
     auto load_w = [&](uint4 (&wb)[MAXS], int q) {
         const bool live = q < n_sub;                    // the same for the whole workgroup
-        const uint32_t row = live ? (uint32_t)((size_t)(tile_of(live ? q : 0) * 16 + li) * K * 2) : 0u;
+        // a tile starts at 16 K t either way; a weight row beyond N lies beyond the descriptor's end
+        const uint32_t row = live ? (uint32_t)((size_t)tile_of(live ? q : 0) * 16 * K * 2) : 0u;
 #pragma unroll
         for (int s = 0; s < MAXS; ++s)
             wb[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
@@ -811,8 +824,9 @@ SOC_EXPORT int soc_gemm_sweep_plan(int N, int K, int swiglu, int* n_waves, int* 
 // up to 32 must not exceed 256. The matrices lie below 4 GiB.
 SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
                                    int mode, int n_waves, int workgroups, const float* ssq_in, int ssq_tiles,
-                                   int norm_dim, float eps, hipStream_t stream) {
+                                   int norm_dim, float eps, int w_tiled, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || !C) return (int)hipErrorInvalidValue;
     if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > 16 || workgroups < 1) return (int)hipErrorInvalidValue;
@@ -831,7 +845,7 @@ SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M,
     const int steps = pl.k_per_wave / 32;
 #define SOC_SW(TC_, MODE_, MAXS_) \
     hipLaunchKernelGGL((gemm_bf16_sweep_kernel<TC_, MODE_, MAXS_>), grid, block, 0, stream, (const bf16*)X, \
-                       (const bf16*)W, (TC_*)C, M, N, K, pl, nm)
+                       (const bf16*)W, (TC_*)C, M, N, K, pl, nm, w_tiled)
 #define SOC_SW_STEPS(TC_, MODE_)                                                           \
     do {                                                                                   \
         if (steps <= 2) SOC_SW(TC_, MODE_, 2); else if (steps <= 4) SOC_SW(TC_, MODE_, 4); \

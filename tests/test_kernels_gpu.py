@@ -268,6 +268,52 @@ def test_sweep_form_of_the_skinny_products(kernel_sets, M, d, K):
         torch.testing.assert_close(got[name].float(), want[name].float(), **tol)
 
 
+@pytest.mark.parametrize("M,d,K", [(1, 64, 64), (8, 2560, 4096), (16, 80, 224), (5, 2560, 9728), (3, 4096, 96),
+                                   (16, 6144, 2560), (9, 48, 32)])
+def test_weights_by_tile_give_the_same_bits(kernel_sets, M, d, K):
+    """Products of at most 16 rows read a copy of their weight laid out by tile. The sums are
+    added in the same order as from the rows, so every form of product returns the same
+    bits either way; a weight changed in place is copied anew; sizes that do not tile, and
+    products of more rows, read the rows."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    y, w = rnd((M, K), torch.bfloat16, 60), rnd((d, K), torch.bfloat16, 61, K ** -0.5)
+    res = rnd((M, d), torch.float32, 62)
+    gain = (1 + 0.3 * torch.randn(d)).to(DEV)
+    w2 = rnd((6144 if d > 1000 else 336, d), torch.bfloat16, 63, d ** -0.5)
+    ff = 9728 if d > 1000 else 160
+    wgu = rnd((2 * ff, d), torch.bfloat16, 64, d ** -0.5)
+    kept = (hip.pack_weights, hip.pack_min_elements, hip.sweep_rows, hip.sweep_min_items, hip.addnorm_splits)
+
+    def run(pack, sweep, splits):
+        hip.pack_weights, hip.pack_min_elements = pack, 0
+        hip.sweep_rows, hip.sweep_min_items = (1, 1) if sweep else (0, 1)
+        hip.addnorm_splits = splits
+        hip.forget_packed()
+        out = [hip.linear(y, w), hip.linear(y, w, out_dtype=torch.float32)]
+        r = res.clone()
+        owed = hip.linear_add_norm(y, w, r, gain, 1e-6)
+        out += [r, owed.x, owed.ssq[:, :(d + 15) // 16].clone()]
+        if d % 32 == 0:
+            out += [hip.linear(owed, w2), hip.linear_swiglu(owed, wgu, 16), hip.linear_swiglu(owed.x, wgu, 16)]
+        assert bool(hip._packed) == pack
+        return out
+
+    try:
+        for sweep in (False, True):
+            for splits in (1, 2):
+                by_row, by_tile = run(False, sweep, splits), run(True, sweep, splits)
+                for a, b in zip(by_row, by_tile):
+                    assert torch.equal(a, b)
+        before = hip.linear(y, w)
+        w.mul_(2)
+        assert torch.equal(hip.linear(y, w).float(), 2 * before.float())         # the copy followed the weight
+        odd = rnd((d + 8, K), torch.bfloat16, 65)
+        assert hip._by_tile(odd)[1] == 0 and hip._by_tile(odd[:d])[1] == 1
+    finally:
+        hip.pack_weights, hip.pack_min_elements, hip.sweep_rows, hip.sweep_min_items, hip.addnorm_splits = kept
+        hip.forget_packed()
+
+
 def test_linear_float32_is_not_reduced_precision(kernel_sets):
     """Values that bfloat16 or a 19-bit matrix mode would round away survive."""
     hip, _ = kernel_sets[torch.float32]
