@@ -677,9 +677,11 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
 // weight tiles g, g + G, g + 2 G, ...: per tile a wave loads only weights, multiplies, and
 // leaves its sums in LDS, where the first four waves add them and do the epilogue while the
 // others go on. The weights of two tiles are on their way at any time, and x is read once per
-// workgroup. At one row the form of a workgroup per tile streams the weights 8 % faster; from
-// 3 rows on this one wins (gate+up of a 4B-sized layer at 8 rows: 23.3 against 27.0 us, at 16
-// rows 24.8 against 33.8 us; the output head of 151,936 rows at 8 rows: 141 against 169 us).
+// workgroup. With the weights row by row, the form of a workgroup per tile streams them 8 %
+// faster at one row and this one wins from 3 rows on (gate+up of a 4B-sized layer at 8 rows:
+// 23.3 against 27.0 us, at 16 rows 24.8 against 33.8 us; the output head of 151,936 rows at 8
+// rows: 141 against 169 us); with the weights by tile it wins at every number of rows
+// (gate+up 19.7 us at 8 rows).
 // SWIGLU: an item is a pair of tiles (gate rows, then up rows of the same 16 outputs), swept
 // one after the other; the gate sums wait in registers for the up sums.
 // (The form with a residual epilogue stays with the kernel above: its few tiles with a long K

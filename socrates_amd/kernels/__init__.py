@@ -152,10 +152,11 @@ class HipKernels:
         # The sweep form of the skinny product (one workgroup per compute unit keeps its slices
         # of x in registers and walks over the weight tiles): from this many rows of x on, for
         # products of at least ``sweep_min_items`` weight tiles (pairs of them with SwiGLU).
-        # Measured on an MI355X at 4B-sized layers: at one row it streams the weights 8 % slower
-        # than a workgroup per tile, at two rows a decode step takes the same time either way,
-        # from three rows on it wins, by a quarter at 16 rows.
-        self.sweep_rows = 3             # 0: never
+        # Measured on an MI355X at 4B-sized layers with the weights laid out by tile: a decode
+        # step of one request takes 2.42 ms with it and 2.52 ms without, of 8 requests 2.87
+        # against 3.2 ms, of 16 requests 3.66 against 4.3 ms. (With the weights row by row it
+        # lost at one row and won from three on.)
+        self.sweep_rows = 1             # 0: never
         self.sweep_min_items = 256
         # Products of at most 16 rows read a second copy of their weight, laid out by tile
         # ([N / 16, K / 32, 16, 32]: a wave's load of 16 rows x 32 k is 1 KB in one piece instead
