@@ -308,20 +308,31 @@ class HipKernels:
         graph is being captured: such a call reads the weight row by row); the entry keeps the
         weight alive, so its address cannot come to mean another tensor."""
         N, K = w.shape
-        if (not self.pack_weights or N % 16 or K % 32 or N * K < self.pack_min_elements
-                or w.dtype != torch.bfloat16 or not w.is_contiguous()):
+        if N % 16 or K % 32 or w.dtype != torch.bfloat16 or not w.is_contiguous():
             return w, 0
         key = (w.data_ptr(), N, K)
         entry = self._packed.get(key)
-        if entry is None or entry[2] != w._version:         # (a weight written to in place is copied anew)
-            if torch.cuda.is_current_stream_capturing():
-                return w, 0
+        if entry is not None and entry[2] == w._version:
+            return entry[1], 1
+        # (a weight written to in place is copied anew)
+        if (not self.pack_weights or N * K < self.pack_min_elements or torch.cuda.is_current_stream_capturing()):
+            return w, 0
+        try:
             tiled = w.view(N // 16, 16, K // 32, 32).permute(0, 2, 1, 3).contiguous()
-            entry = self._packed[key] = (w, tiled, w._version)
-        return entry[1], 1
+        except torch.cuda.OutOfMemoryError:
+            # no room for second copies (weights and cache fill the GPU): no new ones from now
+            # on; the weights that have one keep using it
+            import warnings
+            warnings.warn("no memory for a copy of a weight laid out by tile; products of few rows read the "
+                          "rows of the weights that have none (HipKernels.pack_weights = False says so up front)")
+            self.pack_weights = False
+            return w, 0
+        self._packed[key] = (w, tiled, w._version)
+        return tiled, 1
 
     def forget_packed(self) -> None:
-        """Drop the copies by tile (after weights were changed in place, or to free memory)."""
+        """Drop the copies by tile (to free memory). Graphs captured with this kernel set read
+        the copies by address: drop those first and capture anew afterwards."""
         self._packed.clear()
 
     def _sweep_plan(self, M, N, K, swiglu=False):
