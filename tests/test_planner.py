@@ -1,4 +1,8 @@
-"""The host arithmetic that plans launches: key splits of the MFMA attention kernel."""
+"""The host arithmetic that plans launches: key splits of the MFMA attention kernel, and the
+workgroups of a product's sweep over its weight tiles."""
+
+import ctypes
+from ctypes import c_int
 
 import pytest
 
@@ -32,3 +36,31 @@ def test_key_splits_cases_that_used_to_exceed_the_limit():
     # a short context is not cut below 64 keys, a full launch is not cut at all
     assert plan_key_splits(1, 8, 4, 100)[1] <= 4
     assert plan_key_splits(128, 8, 4, 4096) == (4096, 1)
+
+
+def test_a_sweep_shares_the_tiles_out_evenly():
+    """At most one workgroup per compute unit (256), every workgroup the same number of weight
+    tiles (tile pairs with SwiGLU) up to one, no workgroup without a tile; K beyond 16 waves
+    of 8 steps of 32 is refused. (The plan is host code of the product library; calling it
+    needs the library, not a GPU.)"""
+    from socrates_amd.kernels.build import load_library
+    lib = load_library("gemm")
+    lib.soc_gemm_sweep_plan.restype = c_int
+    for swiglu in (0, 1):
+        for N in (32, 64, 4096, 6144, 8192, 19456, 24576, 51200, 151936, 151968):
+            for K in (8, 64, 2560, 4096):
+                nw, wgs = c_int(0), c_int(0)
+                assert lib.soc_gemm_sweep_plan(c_int(N), c_int(K), c_int(swiglu), ctypes.byref(nw), ctypes.byref(wgs)) == 1
+                items = N // 32 if swiglu else (N + 15) // 16
+                assert nw.value == 16 and 1 <= wgs.value <= min(items, 256)
+                most = (items + wgs.value - 1) // wgs.value
+                assert most == (items + 255) // 256                        # as few tiles for the busiest as 256 units allow
+                assert (most - 1) * wgs.value < items                      # nobody is idle
+    nw, wgs = c_int(0), c_int(0)
+    for K in (4104, 5120, 9728):
+        assert lib.soc_gemm_sweep_plan(c_int(2560), c_int(K), c_int(0), ctypes.byref(nw), ctypes.byref(wgs)) == 0
+    # the shapes of a 4B-sized layer: 608 tile pairs as 203 x 3, 384 tiles as 192 x 2
+    lib.soc_gemm_sweep_plan(c_int(19456), c_int(2560), c_int(1), ctypes.byref(nw), ctypes.byref(wgs))
+    assert wgs.value == 203
+    lib.soc_gemm_sweep_plan(c_int(6144), c_int(2560), c_int(0), ctypes.byref(nw), ctypes.byref(wgs))
+    assert wgs.value == 192
