@@ -130,10 +130,11 @@ class Engine:
         awaited, where the scheduler knows it without them (``Scheduler.repeats``): the
         device takes the tokens from the sampler's output, so it goes from one decode step
         into the next without waiting for the host to read, record, plan and launch. Each
-        call still returns with exactly one more step's tokens recorded. A request that stops
-        at a stop token has then one place in the step that was queued ahead; that place's
-        token is dropped, and its key and value lie beyond the request's end in pages that
-        are freed with it."""
+        call still returns with exactly one more step's tokens recorded; between calls the
+        cache manager's lengths (and pages) are then those of the step queued ahead, one
+        token further than the recorded outputs. A request that stops at a stop token has
+        one place in the step that was queued ahead; that place's token is dropped, and its
+        key and value lie beyond the request's end in pages that are freed with it."""
         flight = self._flight
         self._flight = None
         if flight is not None and not any(self._live(p.request) for p in flight.plan):
