@@ -367,7 +367,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
                        float* __restrict__ part_ml, int* __restrict__ arrivals, int Hq, int Hkv, int BS,
                        int bs_shift, float scale, int window, int split_len_arg, int n_splits,
-                       int group_pad_log2, FusedQkv fz) {
+                       int group_pad_log2, FusedQkv fz, int out_tiled) {
     static_assert(!FUSED || (RT == 1 && QK_K32), "the fused form: one row tile, head sizes in steps of 32");
     // One piece of LDS: the waves' V tiles while the keys are walked; afterwards, with key
     // splits, what the four waves of the workgroup have gathered, to be combined.
@@ -530,6 +530,15 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         }
     }
 
+    // Where four outputs of a row go: element `at` = (token * Hq + head) * D + d of out
+    // [N, Hq * D], or (out_tiled: at most 16 tokens) the same element of out [Hq * D / 32, 16, 32],
+    // the layout in which the product that follows reads 64 bytes of every row side by side.
+    auto out_at = [&](size_t at) -> bf16* {
+        if (!out_tiled) return out + at;
+        const size_t width = (size_t)Hq * D, tok = at / width;
+        const int col = (int)(at - tok * width);
+        return out + ((size_t)(col / 32) * 16 + tok) * 32 + col % 32;
+    };
     f32x4_t o[RT][DV];
     float m[RT], l[RT];
 #pragma unroll
@@ -765,7 +774,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 uint2 pk;
                 pk.x = pack_bf16x2(o[rt][j][0] * inv, o[rt][j][1] * inv);
                 pk.y = pack_bf16x2(o[rt][j][2] * inv, o[rt][j][3] * inv);
-                *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
+                *reinterpret_cast<uint2*>(out_at(row_q[rt] + j * 16 + 4 * kb)) = pk;
             }
         }
         return;
@@ -812,7 +821,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 uint2 pk;
                 pk.x = pack_bf16x2(a.x * inv, a.y * inv);
                 pk.y = pack_bf16x2(a.z * inv, a.w * inv);
-                *reinterpret_cast<uint2*>(out + row_q[rt] + j * 16 + 4 * kb) = pk;
+                *reinterpret_cast<uint2*>(out_at(row_q[rt] + j * 16 + 4 * kb)) = pk;
             } else {
                 // written through the caches (agent scope): another workgroup reads it below
                 float* dst = part_o + pi * D + j * 16 + 4 * kb;
@@ -901,7 +910,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             uint2 pk;
             pk.x = pack_bf16x2(acc.x * inv, acc.y * inv);
             pk.y = pack_bf16x2(acc.z * inv, acc.w * inv);
-            *reinterpret_cast<uint2*>(out + row * D + e4 * 4) = pk;
+            *reinterpret_cast<uint2*>(out_at(row * D + e4 * 4)) = pk;
         }
     }
 }
@@ -917,14 +926,17 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 // tokens per block (the blocks may cover some of the N tokens only; the others' outputs are
 // not touched), and `arrivals`, one int per task (row block x kv head x chunk of 16 heads),
 // zero before the call and zero again after it; calls that may run at the same time need
-// arrival counts of their own.
+// arrival counts of their own. out_tiled (N <= 16, Hq * D a multiple of 32): out is written
+// [Hq * D / 32, 16, 32] instead of [N, Hq * D], for a product that reads its x by tile.
 SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const void* v_pool,
                                         const int* block_table, int table_width, const int* token_rows,
                                         const int* positions, const int* row_blocks, int n_row_blocks,
                                         void* out, float* part_o, float* part_ml, int* arrivals, int N,
                                         int Hq, int Hkv, int BS, float scale, int window, int split_len,
-                                        int n_splits, int row_tiles, int group_pad_log2, hipStream_t stream) {
+                                        int n_splits, int row_tiles, int group_pad_log2, int out_tiled,
+                                        hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
+    if (out_tiled && (N > 16 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
         return (int)hipErrorInvalidValue;
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
@@ -943,7 +955,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
         for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
-        scale, window, split_len, n_splits, group_pad_log2, fz
+        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled
     // Row tiles beyond what the registers hold at this head size are refused: two up to head
     // size 128, four up to 64.
     const bool tp = bs_shift >= 4;
@@ -984,11 +996,12 @@ SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, 
                                                 int Hkv, int BS, float scale, int window, int split_len,
                                                 int n_splits, int group_pad_log2, const float* q_gain,
                                                 const float* k_gain, const float* rope_table, float eps,
-                                                int write_kv, hipStream_t stream) {
+                                                int write_kv, int out_tiled, hipStream_t stream) {
     if constexpr (!QK_K32) {
         return (int)hipErrorNotSupported;
     } else {
         if (N <= 0) return 0;
+        if (out_tiled && (N > 16 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
         if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
             return (int)hipErrorInvalidValue;
         if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;
@@ -1011,7 +1024,7 @@ SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, 
             for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_FUSED_ARGS (const bf16*)nullptr, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, (const int*)nullptr, N, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
-        scale, window, split_len, n_splits, group_pad_log2, fz
+        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled
         if (bs_shift >= 4)
             hipLaunchKernelGGL((paged_attn_mfma_kernel<1, true, true>), grid, dim3(256), 0, stream, SOC_FUSED_ARGS);
         else

@@ -240,6 +240,7 @@ struct SkNorm {
     int* split_count;           // the same: [tiles], zero before the launch and after it
 };
 constexpr int SK_SWIGLU = 1, SK_SCALED = 2, SK_ADDNORM = 4;
+constexpr int SK_W_TILED = 1, SK_X_TILED = 2, SK_C_TILED = 4;     // the `layout` argument of the entry points
 constexpr int SK_SSQ_MAX_PAIRS = 16 * 16;       // 16 rows x 16 segments of 256 tiles: norms over up to 65,536 elements
 
 // SCALED: the factor of each of the 16 rows, from the partial sums of squares ssq [M, stride]
@@ -314,7 +315,7 @@ template <typename TC, int MT, int RW, int MODE = 0>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, RW, MODE))
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
-                        int k_per_wave, SkNorm nm, int w_tiled = 0) {
+                        int k_per_wave, SkNorm nm, int layout = 0) {
     constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED, ADDNORM = MODE & SK_ADDNORM;
     static_assert(!(SCALED || ADDNORM) || (MT == 1 && RW == 1), "the norm forms take one tile of each");
     __shared__ float red[sk_max_waves(MT, RW, MODE) * MT * RW * 256];
@@ -334,8 +335,13 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     // The weights lie row by row, [N, K], or by tile (w_tiled: [N / 16, K / 32, 16, 32], N a
     // multiple of 16 and K of 32): a wave's load of 16 rows x 32 k is then 1 KB in one piece
     // instead of sixteen pieces of 64 bytes. Either way a tile of 16 rows starts at 16 K t.
+    // x (at most 16 rows, the norm forms) and the SwiGLU form's output may lie by tile too,
+    // [K / 32, 16, 32] with the rows from M on never written or read: what such a product
+    // hands to the next one is then read in pieces of M x 64 bytes instead of M pieces.
+    const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED, c_tiled = layout & SK_C_TILED;
     const int w_rs = w_tiled ? 32 : K;              // elements from a row of a tile to the next
     const int w_ss = w_tiled ? 512 : 32;            // elements from a step of 32 k to the next
+    const int x_rs = x_tiled ? 32 : K, x_ss = x_tiled ? 512 : 32;
     // Element offsets of this lane's rows (offsets, not pointers: the loads stay global
     // loads); a row outside the matrix is never loaded.
     size_t w_off[RW];
@@ -348,11 +354,13 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     // X is read through a buffer descriptor that covers its M rows: a lane whose row lies
     // outside (M = 8 leaves half of the 16 lanes of a tile without one) gets zeros and asks
     // memory for nothing. X comes from L2 for every workgroup, so this halves that traffic.
+    const int x_bytes = x_tiled ? K * 32 : M * K * 2;
     const __amdgpu_buffer_rsrc_t x_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, M * K * 2, 0x00020000);
-    uint32_t x_off[MT];                                  // bytes
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, x_bytes, 0x00020000);
+    uint32_t x_off[MT];                                  // bytes; by tile a row from M on starts where the buffer ends
 #pragma unroll
-    for (int t = 0; t < MT; ++t) x_off[t] = (uint32_t)(((t * 16 + li) * K + lk) * 2);
+    for (int t = 0; t < MT; ++t)
+        x_off[t] = x_tiled && t * 16 + li >= M ? (uint32_t)x_bytes : (uint32_t)(((t * 16 + li) * x_rs + lk) * 2);
     f32x4 acc[MT][RW];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
@@ -380,7 +388,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
             B.w[r][u] = *reinterpret_cast<const uint4*>(W + w_off[r] + (size_t)((K0) / 32 + u) * w_ss); \
         _Pragma("unroll") for (int t = 0; t < MT; ++t)                                               \
             B.x[t][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(              \
-                x_rsrc, x_off[t] + (uint32_t)(((K0) + 32 * u) * 2), 0, 0));                          \
+                x_rsrc, x_off[t] + (uint32_t)(((K0) / 32 + u) * x_ss * 2), 0, 0));                   \
     }
 #define SK_COMPUTE(B)                                                                               \
     _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u)                                            \
@@ -426,7 +434,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 #pragma unroll
             for (int t = 0; t < MT; ++t)
                 b0.x[t][u] = in ? __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                                      x_rsrc, x_off[t] + (uint32_t)(kk * 2), 0, 0))
+                                      x_rsrc, x_off[t] + (uint32_t)(((kk / 32) * x_ss + kk % 32) * 2), 0, 0))
                                 : make_uint4(0u, 0u, 0u, 0u);
         }
         SK_COMPUTE(b0)
@@ -453,7 +461,9 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
             }
             const int m = ln % 16, col = blockIdx.x * 16 + 4 * (ln / 16) + e;
             if constexpr (SCALED) { const float f = sk_row_factor(nm, norm_part, m); g *= f; u *= f; }
-            if (m < M && 2 * col < N) C[(size_t)m * (N / 2) + col] = from_float<TC>(u * (g / (1.0f + expf(-g))));
+            if (m < M && 2 * col < N)
+                C[c_tiled ? ((size_t)(col / 32) * 16 + m) * 32 + col % 32 : (size_t)m * (N / 2) + col] =
+                    from_float<TC>(u * (g / (1.0f + expf(-g))));
         }
         return;
     }
@@ -528,13 +538,13 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
 
 template <typename TC, int MT, int RW>
 static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N, int K,
-                         int n_waves, int k_splits, int w_tiled, hipStream_t stream) {
+                         int n_waves, int k_splits, int layout, hipStream_t stream) {
     // ranges are multiples of the 128-k step, so only the end of K can be a partial step
     const int k_per_split = ((K + k_splits - 1) / k_splits + SK_STEP - 1) / SK_STEP * SK_STEP;
     const int k_per_wave = ((k_per_split + n_waves - 1) / n_waves + SK_STEP - 1) / SK_STEP * SK_STEP;
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<TC, MT, RW>), dim3((N + 16 * RW - 1) / (16 * RW), k_splits),
                        dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (TC*)C, Cpart, M, N,
-                       K, k_per_split, k_per_wave, SkNorm{}, w_tiled);
+                       K, k_per_split, k_per_wave, SkNorm{}, layout);
     return soc_last_error();
 }
 
@@ -545,9 +555,11 @@ static int launch_skinny(const void* X, const void* W, void* C, float* Cpart, in
 // factor is applied to the sums (the SCALED form above). bfloat16 output only then.
 SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C, int M, int N, int K,
                                            int c_dtype, int n_waves, const float* ssq_in, int ssq_tiles,
-                                           int norm_dim, float eps, int w_tiled, hipStream_t stream) {
+                                           int norm_dim, float eps, int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
+    if ((layout & ~7) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) || ((layout & SK_X_TILED) && K % 32) ||
+        ((layout & SK_C_TILED) && (N % 64 || c_dtype != 1)))
+        return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23) || N % 32) return (int)hipErrorInvalidValue;
     if (n_waves < 2 || n_waves > SK_MAX_WAVES_SWIGLU || n_waves % 2) return (int)hipErrorInvalidValue;
     if (ssq_in && (ssq_tiles < 1 || ssq_tiles > 16 * SK_SSQ_MAX_PAIRS || norm_dim < 1 || c_dtype != 1))
@@ -560,15 +572,15 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
     if (ssq_in)
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU | SK_SCALED>), dim3(N / 32, 1),
                            dim3(n_waves * 64), 0, stream, (const bf16*)X, (const bf16*)W, (bf16*)C,
-                           (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, w_tiled);
+                           (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, layout);
     else if (c_dtype == 0)
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<float, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (float*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave, nm, w_tiled);
+                           k_per_split, k_per_wave, nm, layout);
     else
         hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, SK_SWIGLU>), dim3(N / 32, 1), dim3(n_waves * 64), 0,
                            stream, (const bf16*)X, (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K,
-                           k_per_split, k_per_wave, nm, w_tiled);
+                           k_per_split, k_per_wave, nm, layout);
     return soc_last_error();
 }
 
@@ -585,9 +597,10 @@ SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, 
                                          int n_waves, const float* ssq_in, int ssq_tiles, int norm_dim,
                                          float eps, float* residual, const float* gain, void* x_out,
                                          float* ssq_out, int k_splits, float* split_sums, int* split_count,
-                                         int w_tiled, hipStream_t stream) {
+                                         int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
+    if ((layout & ~3) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) || ((layout & SK_X_TILED) && K % 32))
+        return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > SK_MAX_WAVES_SWIGLU) return (int)hipErrorInvalidValue;
     if (!ssq_in && !residual) return (int)hipErrorInvalidValue;
@@ -605,7 +618,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, 
     const dim3 grid((N + 15) / 16, k_splits), block(n_waves * 64);
 #define SOC_SKN(MODE_) \
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, MODE_>), grid, block, 0, stream, (const bf16*)X, \
-                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, w_tiled)
+                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, layout)
     if (ssq_in && residual) SOC_SKN(SK_SCALED | SK_ADDNORM);
     else if (residual) SOC_SKN(SK_ADDNORM);
     else SOC_SKN(SK_SCALED);
@@ -635,13 +648,16 @@ SOC_EXPORT void soc_gemm_skinny_plan(int M, int N, int K, int allow_split, int* 
 }
 
 // M <= 64, K a multiple of 8. k_splits == 1: C [M, N] in c_dtype. k_splits > 1: float32
-// partial sums Cpart [k_splits, M, N] (C is not written). w_tiled (here and in the entry
-// points around): W lies by tile, [N / 16, K / 32, 16, 32], N a multiple of 16 and K of 32.
+// partial sums Cpart [k_splits, M, N] (C is not written). layout (here and in the entry
+// points around): SK_W_TILED, W lies by tile, [N / 16, K / 32, 16, 32], N a multiple of 16 and
+// K of 32; SK_X_TILED, x (at most 16 rows) lies [K / 32, 16, 32], rows from M on never read;
+// SK_C_TILED (SwiGLU forms, bfloat16), the output is written that way.
 SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float* Cpart, int M, int N,
                                     int K, int c_dtype, int row_tiles, int n_waves, int k_splits,
-                                    int w_tiled, hipStream_t stream) {
+                                    int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
+    if ((layout & ~3) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) || ((layout & SK_X_TILED) && (K % 32 || M > 16)))
+        return (int)hipErrorInvalidValue;
     if (M > 64 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;   // 32-bit byte offsets into X
     if (n_waves < 1 || n_waves > (M <= 16 && row_tiles == 1 ? SK_MAX_WAVES_SWIGLU : SK_MAX_WAVES) || k_splits < 1 ||
         k_splits > 65535)
@@ -650,7 +666,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
     const int MT = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     if (row_tiles != 2 && !((row_tiles == 4 || row_tiles == 1) && MT == 1)) return (int)hipErrorInvalidValue;
 #define SOC_SK(TC_, MT_, RW_) \
-    return launch_skinny<TC_, MT_, RW_>(X, W, C, Cpart, M, N, K, n_waves, k_splits, w_tiled, stream)
+    return launch_skinny<TC_, MT_, RW_>(X, W, C, Cpart, M, N, K, n_waves, k_splits, layout, stream)
     if (c_dtype == 0) {
         if (MT == 1 && row_tiles == 4) SOC_SK(float, 1, 4);
         if (MT == 1 && row_tiles == 1) SOC_SK(float, 1, 1);
@@ -697,8 +713,9 @@ struct SwPlan {
 template <typename TC, int MODE, int MAXS>
 __global__ void __launch_bounds__(1024)
 gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C, int M,
-                       int N, int K, SwPlan pl, SkNorm nm, int w_tiled) {
+                       int N, int K, SwPlan pl, SkNorm nm, int layout) {
     constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED;
+    const bool w_tiled = layout & SK_W_TILED, c_tiled = layout & SK_C_TILED;
     static_assert(!(MODE & SK_ADDNORM), "the residual epilogue stays with the skinny kernel");
     constexpr int SUB = SWIGLU ? 2 : 1;
     __shared__ __attribute__((aligned(16))) float red[2][16 * 256];     // [tile parity][wave][lane][4]
@@ -784,7 +801,9 @@ gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, T
         if constexpr (SWIGLU) {
             if (q % 2 == 0) { held = sum; return; }
             const int col = (tile / 2) * 16 + rc, half = N / 2;
-            if (rm < M && col < half) C[(size_t)rm * half + col] = from_float<TC>(sum * (held / (1.0f + expf(-held))));
+            if (rm < M && col < half)
+                C[c_tiled ? ((size_t)(col / 32) * 16 + rm) * 32 + col % 32 : (size_t)rm * half + col] =
+                    from_float<TC>(sum * (held / (1.0f + expf(-held))));
         } else {
             const int n = tile * 16 + rc;
             if (rm < M && n < N) C[(size_t)rm * N + n] = from_float<TC>(sum);
@@ -826,9 +845,11 @@ SOC_EXPORT int soc_gemm_sweep_plan(int N, int K, int swiglu, int* n_waves, int* 
 // up to 32 must not exceed 256. The matrices lie below 4 GiB.
 SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
                                    int mode, int n_waves, int workgroups, const float* ssq_in, int ssq_tiles,
-                                   int norm_dim, float eps, int w_tiled, hipStream_t stream) {
+                                   int norm_dim, float eps, int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (w_tiled && (N % 16 || K % 32)) return (int)hipErrorInvalidValue;
+    if ((layout & ~5) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) ||
+        ((layout & SK_C_TILED) && (!(mode & SK_SWIGLU) || N % 64)))
+        return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || !C) return (int)hipErrorInvalidValue;
     if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > 16 || workgroups < 1) return (int)hipErrorInvalidValue;
@@ -847,7 +868,7 @@ SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M,
     const int steps = pl.k_per_wave / 32;
 #define SOC_SW(TC_, MODE_, MAXS_) \
     hipLaunchKernelGGL((gemm_bf16_sweep_kernel<TC_, MODE_, MAXS_>), grid, block, 0, stream, (const bf16*)X, \
-                       (const bf16*)W, (TC_*)C, M, N, K, pl, nm, w_tiled)
+                       (const bf16*)W, (TC_*)C, M, N, K, pl, nm, layout)
 #define SOC_SW_STEPS(TC_, MODE_)                                                           \
     do {                                                                                   \
         if (steps <= 2) SOC_SW(TC_, MODE_, 2); else if (steps <= 4) SOC_SW(TC_, MODE_, 4); \

@@ -17,7 +17,7 @@ import torch
 
 from .build import KernelBuildError, build_all, compile_library, load_library
 
-__all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "NormOwed", "build_all",
+__all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "NormOwed", "RowsByTile", "build_all",
            "compile_library", "load_library", "plan_key_splits"]
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -60,9 +60,9 @@ _GEMM_SIGNATURES = {
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
-    "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, P],
+    "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
-    "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, P],
+    "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, I, P],
     "soc_attention_head_dim": [],
 }
 
@@ -107,6 +107,28 @@ class NormOwed:
     @property
     def shape(self):
         return self.x.shape
+
+
+class RowsByTile:
+    """At most 16 rows of bfloat16 activations laid out by tile, ``data`` [dim / 32, 16, 32]
+    (element (row, col) at [col // 32, row, col % 32]; rows from ``rows`` on are never written
+    or read), for the product that takes them next: it then asks the L2 for one piece of
+    rows x 64 bytes per load where rows laid out one after the other give it that many pieces.
+    Made by ``decode_attention`` and ``linear_swiglu`` where the caller allows it (``by_tile``:
+    the caller hands the result to ``linear_add_norm`` or ``linear`` and nowhere else), taken
+    by those two."""
+    __slots__ = ("data", "rows", "dim")
+
+    def __init__(self, data, rows, dim):
+        self.data, self.rows, self.dim = data, rows, dim
+
+    @property
+    def shape(self):
+        return (self.rows, self.dim)
+
+    def by_rows(self):
+        """The rows as an ordinary [rows, dim] tensor (a copy)."""
+        return self.data[:, :self.rows].permute(1, 0, 2).reshape(self.rows, self.dim)
 
 
 class HipKernels:
@@ -166,6 +188,10 @@ class HipKernels:
         # is no multiple of 16 or K of 32, are read row by row.
         self.pack_weights = True
         self.pack_min_elements = 1 << 20
+        # what a decode step's attention and gate / up product hand to the projection behind
+        # them may lie by tile too (``RowsByTile``); measured: 0.8 and 0.6 us less for O and
+        # down of a 4B-sized layer at 8 rows, 1.9 and 1.5 us at 16
+        self.rows_by_tile = True
         self._packed = {}               # (address, N, K) -> (the weight, its copy by tile, the weight's version)
         # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
@@ -271,9 +297,11 @@ class HipKernels:
                                    c_int(self.code), self._stream()), "swiglu")
         return out
 
-    def linear_swiglu(self, x, w_gate_up, interleave=0):
+    def linear_swiglu(self, x, w_gate_up, interleave=0, by_tile=False):
         """swiglu(x @ w_gate_up^T). With rows interleaved in blocks of 16 and at most 16 rows of
-        x in bfloat16, one kernel: the skinny product applies silu(gate) * up in its epilogue."""
+        x in bfloat16, one kernel: the skinny product applies silu(gate) * up in its epilogue.
+        ``by_tile``: the caller hands the result to ``linear_add_norm`` or ``linear`` only, so
+        it may come as a ``RowsByTile``."""
         owed = x if isinstance(x, NormOwed) else None
         if owed is not None:
             x = owed.x
@@ -283,11 +311,14 @@ class HipKernels:
                 and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N % 32 == 0):
             self._want(x, "x")
             self._want(w_gate_up, "weight", None, (N, K))
-            out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
+            tiled_out = bool(by_tile and self.rows_by_tile and N % 64 == 0)
+            out = torch.empty((N // 64, 16, 32) if tiled_out else (M, N // 2), dtype=self.dtype, device=self.device)
+            result = RowsByTile(out, M, N // 2) if tiled_out else out
             plan = self._sweep_plan(M, N, K, swiglu=True)
             if plan is not None:
-                self._sweep(plan, x, w_gate_up, out, self._SK_SWIGLU, self._owed_args(owed, M, K), what="linear_swiglu")
-                return out
+                self._sweep(plan, x, w_gate_up, out, self._SK_SWIGLU, self._owed_args(owed, M, K), what="linear_swiglu",
+                            layout=4 if tiled_out else 0)
+                return result
             n_waves = self.swiglu_waves          # half of them per tile (gate, up), splitting K
             while n_waves > 2 and K // (n_waves // 2) < 128:
                 n_waves //= 2
@@ -295,9 +326,10 @@ class HipKernels:
             wt, tiled = self._by_tile(w_gate_up)
             _check(self._gemm.soc_gemm_bf16_skinny_swiglu(_ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N),
                                                           c_int(K), c_int(self.code), c_int(n_waves),
-                                                          ssq, c_int(tiles), c_int(dim), c_float(eps), c_int(tiled),
+                                                          ssq, c_int(tiles), c_int(dim), c_float(eps),
+                                                          c_int(tiled | (4 if tiled_out else 0)),
                                                           self._stream()), "linear_swiglu")
-            return out
+            return result
         return self.swiglu(self.linear(owed if owed is not None else x, w_gate_up), interleave)
 
     _SK_SWIGLU, _SK_SCALED = 1, 2
@@ -348,7 +380,7 @@ class HipKernels:
             return None
         return nw.value, wgs.value
 
-    def _sweep(self, plan, x, w, out, mode, owed_args=(None, 0, 0, 0.0), what="linear"):
+    def _sweep(self, plan, x, w, out, mode, owed_args=(None, 0, 0, 0.0), what="linear", layout=0):
         (M, K), N = x.shape, w.shape[0]
         ssq, tiles, dim, eps = owed_args
         if ssq is not None:
@@ -356,7 +388,8 @@ class HipKernels:
         wt, tiled = self._by_tile(w)
         _check(self._gemm.soc_gemm_bf16_sweep(
             _ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(_DTYPE_CODE[out.dtype]), c_int(mode),
-            c_int(plan[0]), c_int(plan[1]), ssq, c_int(tiles), c_int(dim), c_float(eps), c_int(tiled), self._stream()),
+            c_int(plan[0]), c_int(plan[1]), ssq, c_int(tiles), c_int(dim), c_float(eps), c_int(tiled | layout),
+            self._stream()),
             f"{what} (sweep) [{M}x{K}] x [{N}x{K}]^T")
 
     def _owed_args(self, owed, M, K):
@@ -375,13 +408,19 @@ class HipKernels:
         16 rows it is one kernel: the product's epilogue adds to the residual and leaves the
         rows as a NormOwed, whose factor the next product applies (``y`` may be one itself)."""
         owed = y if isinstance(y, NormOwed) else None
-        yx = owed.x if owed is not None else y
-        (M, K), N = yx.shape, w.shape[0]
+        tiled_y = y if isinstance(y, RowsByTile) else None
+        yx = owed.x if owed is not None else (tiled_y.data if tiled_y is not None else y)
+        (M, K), N = (tiled_y.shape if tiled_y is not None else yx.shape), w.shape[0]
         if not (self.dtype == torch.bfloat16 and yx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
                 and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N <= 65536 and self.fuse_norms):
             # (65,536: the sums of squares of a row are summed by one wave per 256 tiles of 16)
             return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps)
-        self._want(yx, "y")
+        if tiled_y is not None:
+            self._want(yx, "y", torch.bfloat16, (K // 32, 16, 32))
+            yx_layout = 2
+        else:
+            self._want(yx, "y", None, (M, K))
+            yx_layout = 0
         self._want(w, "weight", None, (N, K))
         self._want(residual, "residual", torch.float32, (M, N))
         self._want(gain, "norm weight", torch.float32, (N,))
@@ -406,7 +445,7 @@ class HipKernels:
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(yx), _ptr(wt), None, c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(in_tiles),
             c_int(dim), c_float(in_eps), _ptr(residual), _ptr(gain), _ptr(x_out), _ptr(ssq_out),
-            c_int(k_splits), _ptr(sums), _ptr(count), c_int(tiled), self._stream()),
+            c_int(k_splits), _ptr(sums), _ptr(count), c_int(tiled | yx_layout), self._stream()),
             f"linear_add_norm [{M}x{K}] x [{N}x{K}]^T")
         return NormOwed(x_out, ssq_out, N, eps)
 
@@ -479,6 +518,8 @@ class HipKernels:
         skinny kernel then spreads a narrow output over more workgroups."""
         if isinstance(x, NormOwed):
             return self._linear_owed(x, w, out_dtype or self.dtype, n_waves)
+        if isinstance(x, RowsByTile):
+            x = x.by_rows()
         self._want(x, "x")
         self._want(w, "weight")
         if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -749,7 +790,7 @@ class HipKernels:
             c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
             c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(self._split_count), c_int(N),
             c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
-            c_int(rt), c_int(gpl), self._stream()), "paged_attention (mfma)")
+            c_int(rt), c_int(gpl), c_int(0), self._stream()), "paged_attention (mfma)")
 
     def rope_table(self, inv_freq, first_pos, n_pos, out=None):
         """Cosines and sines of positions first_pos .. first_pos + n_pos - 1 with the rotation
@@ -764,14 +805,16 @@ class HipKernels:
         return out
 
     def decode_attention(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps, rope_table, slot, ctx, scale,
-                         window=None, write=True):
+                         window=None, write=True, by_tile=False):
         """A decode step's attention straight from the QKV product's rows: per-head norm,
         rotation, the write of the new key and value, and the attention over the pages in one
         kernel. ``qkv`` [N, (Hq + 2 Hkv) D] (with ``write``) or [N, Hq D]. Returns [N, Hq D],
         or None where this form does not apply (the caller then runs the kernels one after
         the other): bfloat16 steps in which every request brings one token, head sizes in
         steps of 32 without a rotation, in steps of 64 with one (``rope_table``, over the whole
-        head: a lane's slices of a head then hold both partners of every rotated pair)."""
+        head: a lane's slices of a head then hold both partners of every rotated pair).
+        ``by_tile``: the caller hands the result to ``linear_add_norm`` or ``linear`` only, so up
+        to 16 rows may come as a ``RowsByTile``."""
         if not (self.fuse_rope and self.dtype == torch.bfloat16 and self.attention_mfma
                 and getattr(ctx, "max_q_len", 0) == 1 and D % 32 == 0 and 32 <= D <= 256
                 and (rope_table is None or D % 64 == 0) and slot is not None):
@@ -809,16 +852,17 @@ class HipKernels:
                 return None
             part_o = torch.empty((N, Hq, n_splits // 4, D), dtype=torch.float32, device=self.device)
             part_ml = torch.empty((N, Hq, n_splits // 4, 2), dtype=torch.float32, device=self.device)
-        out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
+        tiled = bool(by_tile and self.rows_by_tile and N <= 16 and (Hq * D) % 32 == 0)
+        out = torch.empty((Hq * D // 32, 16, 32) if tiled else (N, Hq * D), dtype=self.dtype, device=self.device)
         self.last_attention_kernel = ("fused", 1)
         _check(lib.soc_paged_attention_decode_fused(
             _ptr(qkv), c_int(heads), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
             c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(out), _ptr(part_o),
             _ptr(part_ml), _ptr(self._split_count), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
             c_float(scale), c_int(int(window) if window else 0), c_int(split_len), c_int(n_splits), c_int(gpl),
-            _ptr(q_gain), _ptr(k_gain), _ptr(rope_table), c_float(eps), c_int(1 if write else 0), self._stream()),
-            "decode_attention")
-        return out
+            _ptr(q_gain), _ptr(k_gain), _ptr(rope_table), c_float(eps), c_int(1 if write else 0),
+            c_int(1 if tiled else 0), self._stream()), "decode_attention")
+        return RowsByTile(out, N, Hq * D) if tiled else out
 
     def paged_attention(self, q, slot, ctx, scale, window=None):
         """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""

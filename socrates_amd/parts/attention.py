@@ -49,6 +49,7 @@ class PagedAttention:
         self.position = (build_part(spec.position, {}, ops)
                          if spec.position is not None else None)
         self.capturable = getattr(self.position, "capturable", True)
+        self._free_layout = {"by_tile": True} if getattr(ops, "rows_by_tile", None) is not None else {}
 
     takes_projection = True     # the block may supply the last product
     takes_norm_owed = True      # x goes to one product only
@@ -68,8 +69,9 @@ class PagedAttention:
             # a decode step: norm, position encoding, cache write and attention in one kernel
             table = self.position.table(ctx.max_ctx_len) if hasattr(self.position, "table") else None
             if self.position is None or table is not None:
+                # (o goes to a product and nowhere else: the kernel set may lay it out as it likes)
                 o = ops.decode_attention(qkv, Hq, s.n_kv_heads, D, self.q_gain, self.k_gain, self.eps, table,
-                                         slot, ctx, s.scale, s.window, write)
+                                         slot, ctx, s.scale, s.window, write, **self._free_layout)
         if o is not None:
             pass
         elif self.position is None or rot is not None:

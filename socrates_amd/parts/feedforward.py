@@ -30,12 +30,14 @@ class SwiGLU:
         else:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
+        # (the activation goes to a product and nowhere else: the kernel set may lay it out as it likes)
+        self._free_layout = {"by_tile": True} if getattr(ops, "rows_by_tile", None) is not None else {}
 
     takes_projection = True     # the block may supply the last product
     takes_norm_owed = True      # x goes to one product only
 
     def forward(self, x, ctx=None, project=None):
-        act = self.ops.linear_swiglu(x, self.w_gate_up, self.interleave)
+        act = self.ops.linear_swiglu(x, self.w_gate_up, self.interleave, **self._free_layout)
         if project is not None:
             return project(act, self.w_down)
         # the block's next norm adds this output to the residual: partial sums are welcome

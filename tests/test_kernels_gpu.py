@@ -295,6 +295,18 @@ def test_weights_by_tile_give_the_same_bits(kernel_sets, M, d, K):
         out += [r, owed.x, owed.ssq[:, :(d + 15) // 16].clone()]
         if d % 32 == 0:
             out += [hip.linear(owed, w2), hip.linear_swiglu(owed, wgu, 16), hip.linear_swiglu(owed.x, wgu, 16)]
+            # what the gate / up product hands on may lie by tile; the projection that takes it
+            # returns the same bits as from rows, and so does any other consumer
+            act = hip.linear_swiglu(owed, wgu, 16, by_tile=True)
+            assert type(act).__name__ == "RowsByTile" and act.shape == (M, ff)
+            assert torch.equal(act.by_rows(), out[-2])
+            w4 = rnd((d, ff), torch.bfloat16, 66, ff ** -0.5)
+            r_rows, r_tile = res.clone(), res.clone()
+            o_rows = hip.linear_add_norm(act.by_rows(), w4, r_rows, gain, 1e-6)
+            o_tile = hip.linear_add_norm(act, w4, r_tile, gain, 1e-6)
+            assert torch.equal(r_rows, r_tile) and torch.equal(o_rows.x, o_tile.x) and torch.equal(o_rows.ssq, o_tile.ssq)
+            assert torch.equal(hip.linear(act, w4), hip.linear(act.by_rows(), w4))
+            out += [r_tile, o_tile.x]
         assert bool(hip._packed) == pack
         return out
 
@@ -448,6 +460,14 @@ def test_decode_attention_from_raw_qkv(kernel_sets, Hq, Hkv, D, bs, norm, rope):
             got_r = hip.decode_attention(qkv[:, :Hq * D].contiguous(), Hq, Hkv, D, q_gain, k_gain, 1e-6, table,
                                          slot_a, ctx, 0.2, window, False)
             close(got_r, want, torch.bfloat16)
+            # the output laid out by tile for the projection behind it: the same bits
+            tiled = hip.decode_attention(qkv[:, :Hq * D].contiguous(), Hq, Hkv, D, q_gain, k_gain, 1e-6, table,
+                                         slot_a, ctx, 0.2, window, False, by_tile=True)
+            if (Hq * D) % 32 == 0:
+                assert type(tiled).__name__ == "RowsByTile" and tiled.shape == (N, Hq * D)
+                assert torch.equal(tiled.by_rows(), got_r)
+            else:
+                assert torch.equal(tiled, got_r)
     hip.attention_splits = None
     assert int(hip._split_count.abs().sum()) == 0
     # where the form does not apply the caller is told so
