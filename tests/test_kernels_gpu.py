@@ -268,6 +268,55 @@ def test_sweep_form_of_the_skinny_products(kernel_sets, M, d, K):
         torch.testing.assert_close(got[name].float(), want[name].float(), **tol)
 
 
+@pytest.mark.parametrize("M,d,K", [(17, 2560, 9728), (64, 2560, 4096), (33, 48, 96), (32, 4096, 12288), (50, 330, 200),
+                                   (64, 5120, 25600), (20, 16, 32)])
+def test_products_of_17_to_64_rows_with_k_split_over_sweeping_workgroups(kernel_sets, M, d, K):
+    """The projection that ends a branch at 17 to 64 rows: partial sums over parts of K, from
+    the weights by tile and row by row (the same bits), against float64; then through
+    ``linear_add_norm`` against the residual sum and norm in float64. Row m of x is scaled by
+    its own factor, so a row that lands in another one's place shows; widths that are no
+    multiple of 16 and K that is no multiple of 32 read the rows."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    y = rnd((M, K), torch.bfloat16, 70) * torch.logspace(-1, 1, M, device=DEV)[:, None].to(torch.bfloat16)
+    w = rnd((d, K), torch.bfloat16, 71, K ** -0.5)
+    kept = (hip.parts_min_k, hip.pack_min_elements, hip.pack_weights)
+    try:
+        hip.parts_min_k, hip.pack_min_elements = 32, 1
+        plan = hip._parts_plan(M, d, K)
+        assert plan is not None and hip._parts_plan(16, d, K) is None and hip._parts_plan(65, d, K) is None
+        exact = y.double() @ w.double().T
+        got = {}
+        for tiles in (True, False):
+            hip.pack_weights = tiles
+            hip.forget_packed()
+            parts = hip.linear(y, w, allow_partial=True)
+            assert parts.dtype == torch.float32 and tuple(parts.shape) == (plan[0], M, d)
+            assert (hip._by_tile(w)[1] == 1) == (tiles and d % 16 == 0 and K % 32 == 0)
+            got[tiles] = parts
+            scale = exact.abs().amax(-1, keepdim=True)
+            assert ((parts.double().sum(0) - exact).abs() / scale).max() < 2e-5 * max(1, K / 512) ** 0.5
+        assert torch.equal(got[True], got[False])
+        hip.pack_weights = True
+        res = rnd((M, d), torch.float32, 72)
+        gain = (1 + 0.3 * torch.randn(d)).to(DEV)
+        r = res.clone()
+        out = hip.linear_add_norm(y, w, r, gain, 1e-6)
+        h = res.double() + exact
+        torch.testing.assert_close(r.double(), h, atol=1e-4 * max(1, K / 512) ** 0.5, rtol=1e-4)
+        close(out, h * torch.rsqrt((h ** 2).mean(-1, keepdim=True) + 1e-6) * gain.double(), torch.bfloat16)
+        # switched off, the same call goes through the library and agrees to a rounding of its bfloat16 output
+        hip.parts_rows, r2 = 0, res.clone()
+        try:
+            assert hip._parts_plan(M, d, K) is None
+            lib_out = hip.linear_add_norm(y, w, r2, gain, 1e-6)
+        finally:
+            hip.parts_rows = 64
+        torch.testing.assert_close(out.float(), lib_out.float(), atol=3e-2, rtol=3e-2)
+    finally:
+        hip.parts_min_k, hip.pack_min_elements, hip.pack_weights = kept
+        hip.forget_packed()
+
+
 @pytest.mark.parametrize("M,d,K", [(1, 64, 64), (8, 2560, 4096), (16, 80, 224), (5, 2560, 9728), (3, 4096, 96),
                                    (16, 6144, 2560), (9, 48, 32)])
 def test_weights_by_tile_give_the_same_bits(kernel_sets, M, d, K):

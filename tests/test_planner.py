@@ -64,3 +64,34 @@ def test_a_sweep_shares_the_tiles_out_evenly():
     assert wgs.value == 203
     lib.soc_gemm_sweep_plan(c_int(6144), c_int(2560), c_int(0), ctypes.byref(nw), ctypes.byref(wgs))
     assert wgs.value == 192
+
+
+def test_parts_of_k_fit_the_registers_and_the_gpu():
+    """The sweep for 17 to 64 rows: every part of K fits what 16 waves hold (5 steps of 32 for
+    up to 32 rows, 3 beyond), parts x groups are at most 256 workgroups, no group is without
+    a tile, and the parts cover K. (Host code of the product library: no GPU needed.)"""
+    from socrates_amd.kernels.build import load_library
+    lib = load_library("gemm")
+    lib.soc_gemm_sweep_parts_plan.restype = c_int
+    for M in (17, 32, 33, 64):
+        for N in (16, 40, 2560, 4096, 5120, 8192):
+            for K in (32, 96, 2048, 4096, 9728, 12288, 25600):
+                parts, kpw, groups = c_int(0), c_int(0), c_int(0)
+                assert lib.soc_gemm_sweep_parts_plan(c_int(M), c_int(N), c_int(K), ctypes.byref(parts),
+                                                     ctypes.byref(kpw), ctypes.byref(groups)) == 1
+                steps, tiles = (K + 31) // 32, (N + 15) // 16
+                per_part = (steps + parts.value - 1) // parts.value
+                assert kpw.value % 32 == 0 and kpw.value // 32 <= (5 if M <= 32 else 3)
+                assert 16 * (kpw.value // 32) >= per_part                  # 16 waves hold a part
+                assert per_part * parts.value >= steps
+                assert 1 <= groups.value <= tiles and parts.value * groups.value <= 256
+                most = (tiles + groups.value - 1) // groups.value
+                assert (most - 1) * groups.value < tiles                   # nobody is idle
+    parts, kpw, groups = c_int(0), c_int(0), c_int(0)
+    for M, N, K in ((65, 2560, 4096), (0, 2560, 4096), (64, 2560, 16)):
+        assert lib.soc_gemm_sweep_parts_plan(c_int(M), c_int(N), c_int(K), ctypes.byref(parts),
+                                             ctypes.byref(kpw), ctypes.byref(groups)) == 0
+    # the projections of a 4B-sized layer at 64 rows: down as 8 parts x 32 groups of 5 tiles
+    lib.soc_gemm_sweep_parts_plan(c_int(64), c_int(2560), c_int(9728), ctypes.byref(parts), ctypes.byref(kpw),
+                                  ctypes.byref(groups))
+    assert (parts.value, kpw.value, groups.value) == (8, 96, 32)
