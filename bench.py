@@ -34,7 +34,7 @@ def preset_dict(name):
     return json.loads(preset_path(name).read_text())
 
 
-def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_, chunk=2048):
+def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_, chunk=2048, block_size=16):
     import torch
 
     from socrates_amd.cache import CacheManager, blocks_for
@@ -50,8 +50,8 @@ def build_engine(cfg_dict, dtype, max_batch, max_len, seed, compile_, chunk=2048
     weights = random_tensors(expected_tensors(plan), seed, dtype=dtype, device="cuda:0")
     model = DecoderModel(plan, weights, ops)
     del weights
-    cache = CacheManager(cache_needs(plan), max_rows=max_batch, max_len=max_len, block_size=16,
-                         num_blocks=max_batch * blocks_for(max_len, 16), dtype=dtype, device="cuda:0")
+    cache = CacheManager(cache_needs(plan), max_rows=max_batch, max_len=max_len, block_size=block_size,
+                         num_blocks=max_batch * blocks_for(max_len, block_size), dtype=dtype, device="cuda:0")
     runner = ModelRunner(model, cache)
     engine = Engine(runner, max_batch=max_batch, max_len=max_len, max_new_tokens=max_len,
                     chunk=chunk, compile=compile_)
@@ -74,6 +74,7 @@ def mixed_workload(args, dtype):
     cfg["num_hidden_layers"] = layers
     rows, portion = args.decode_rows, args.prefill_tokens
     config, engine = build_engine(cfg, dtype, rows + 1, args.max_len, seed=0, compile_=not args.no_graphs,
+                                  block_size=args.block_size,
                                   chunk=portion + rows)
     engine.runner.ops.fuse_norms = not args.no_fused_norms
     if args.dtype == "bf16" and not args.no_tune:
@@ -124,7 +125,7 @@ def mixed_workload(args, dtype):
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "intermediate_size": config.intermediate_size, "vocab_size": config.vocab_size,
                    "requests": args.requests, "new_tokens_per_request": args.new_tokens,
-                   "portion_tokens": portion, "block_size": 16, "hip_graphs": not args.no_graphs},
+                   "portion_tokens": portion, "block_size": args.block_size, "hip_graphs": not args.no_graphs},
         "new_tok_s": round(new / dt, 1), "prompt_tokens": prompt, "new_tokens": new, "seconds": round(dt, 3),
         "preemptions": engine.scheduler.n_preemptions,
     }
@@ -198,6 +199,7 @@ def main(argv=None):
     ap.add_argument("--decode-rows", type=int, default=64, help="--mixed: requests that decode side by side")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
@@ -229,7 +231,8 @@ def main(argv=None):
     sized = {"qwen3-4b": "Qwen3-4B-sized", "qwen3-8b": "Qwen3-8B-sized", "qwen3-32b": "Qwen3-32B-sized"}.get(
         args.preset, args.preset)
     biggest = max(args.batch, 1 if args.no_points else 64)
-    config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs)
+    config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs,
+                                  block_size=args.block_size)
     V = config.vocab_size
     engine.runner.ops.fuse_norms = not args.no_fused_norms
     if args.sweep_rows is not None:
@@ -268,7 +271,7 @@ def main(argv=None):
                    "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "intermediate_size": config.intermediate_size, "vocab_size": V,
                    "tie_word_embeddings": config.tie_word_embeddings, "max_len": args.max_len,
-                   "block_size": 16, "hip_graphs": not args.no_graphs,
+                   "block_size": args.block_size, "hip_graphs": not args.no_graphs,
                    "library_products_tuned": args.dtype == "bf16" and not args.no_tune},
         "prefill": {"value": round(args.prefill_tokens / pre_s, 1), "tokens": args.prefill_tokens,
                     "ms": round(pre_s * 1e3, 3),
