@@ -545,7 +545,8 @@ class HipKernels:
         the weights faster than the library does there); more rows the library product,
         or this package's tiled MFMA kernel if ``library_gemm`` is off. ``allow_partial``: the consumer
         (the residual-add + norm kernel) accepts float32 split-K partial sums [S, M, N]; the
-        skinny kernel then spreads a narrow output over more workgroups."""
+        skinny kernel then spreads a narrow output over more workgroups, and a product of 17 to
+        ``parts_rows`` rows is swept with K split over workgroups instead of going to the library."""
         if isinstance(x, NormOwed):
             return self._linear_owed(x, w, out_dtype or self.dtype, n_waves)
         if isinstance(x, RowsByTile):
