@@ -450,8 +450,16 @@ qk_norm_rope_wide_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out,
     auto load_head = [&](int it) {                         // unconditional: a head outside reads the last one
         return *reinterpret_cast<const uint4*>(qkv + ((size_t)n * heads + min(head_of(it), heads - 1)) * D + e0);
     };
-    uint4 cur = load_head(0);
-    uint4 nxt = load_head(groups > 1 ? 1 : 0);
+    // Heads go in rounds of RD: all loads of a round are issued before the first is used, and
+    // the next round's before this round's work, so a wave of 12 groups of heads pays for two
+    // trips to memory, not for six.
+    constexpr int RD = 6;
+    uint4 cur[RD], nxt[RD];
+    auto load_round = [&](uint4 (&r)[RD], int it0) {
+#pragma unroll
+        for (int j = 0; j < RD; ++j) r[j] = load_head(min(it0 + j, groups - 1));
+    };
+    load_round(cur, 0);
     const int pos = positions ? positions[n] : 0;
     float gq[8], gk[8], cs[8], sn[8];
 #pragma unroll
@@ -469,13 +477,12 @@ qk_norm_rope_wide_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out,
         const int page = block_table[(size_t)token_rows[n] * table_width + pos / BS];
         page_base = ((size_t)page * Hkv * BS + (size_t)(pos % BS)) * D;
     }
-    for (int it = 0; it < groups; ++it) {
-        const uint4 nxt2 = load_head(it + 2 < groups ? it + 2 : groups - 1);       // two loads ahead
+    auto work = [&](const uint4& raw, int it) {
         const int h = head_of(it);
         const bool is_q = h < Hq, is_k = !is_q && h < Hq + Hkv;
         float v[8];
         {
-            const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
         }
@@ -516,8 +523,17 @@ qk_norm_rope_wide_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ q_out,
             *reinterpret_cast<uint4*>(dst + e0) = make_uint4(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]),
                                                              pack_bf16x2(v[4], v[5]), pack_bf16x2(v[6], v[7]));
         }
-        cur = nxt;
-        nxt = nxt2;
+    };
+    for (int it0 = 0; it0 < groups; it0 += RD) {
+        const bool more = it0 + RD < groups;                // the same for the whole wave
+        if (more) load_round(nxt, it0 + RD);
+#pragma unroll
+        for (int j = 0; j < RD; ++j)
+            if (it0 + j < groups) work(cur[j], it0 + j);
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < RD; ++j) cur[j] = nxt[j];
+        }
     }
 }
 
