@@ -206,6 +206,8 @@ def main(argv=None):
     ap.add_argument("--no-tune", action="store_true", help="library products with the library's default choice")
     ap.add_argument("--split-waves", type=int, default=None, help="key splits of the decode attention: waves aimed at")
     ap.add_argument("--split-keys", type=int, default=None, help="key splits of the decode attention: fewest keys of a split")
+    ap.add_argument("--addnorm-splits", type=int, default=None,
+                    help="workgroups that share one tile's K in the projections with a residual epilogue")
     ap.add_argument("--no-fused-norms", action="store_true",
                     help="decode steps with the residual sums and norms in kernels of their own")
     ap.add_argument("--sweep-rows", type=int, default=None,
@@ -241,6 +243,8 @@ def main(argv=None):
         engine.runner.ops.split_target_waves = args.split_waves
     if args.split_keys:
         engine.runner.ops.split_min_keys = args.split_keys
+    if args.addnorm_splits is not None:
+        engine.runner.ops.addnorm_splits = args.addnorm_splits
     if args.dtype == "bf16" and not args.no_tune:
         # the library's products (more than 16 rows): its fastest solution for the prompt's shapes
         # and, up to 16 rows, the faster of the library and this package's own kernel for the timed batch

@@ -461,7 +461,7 @@ class HipKernels:
         while n_waves > 1 and K // n_waves < 128:
             n_waves //= 2
         ssq, in_tiles, dim, in_eps = self._owed_args(owed, M, K)
-        k_splits = self.addnorm_splits or self._addnorm_splits(tiles, K)
+        k_splits = self.addnorm_splits or self._addnorm_splits(tiles, K, M)
         while k_splits > 1 and K // (k_splits * n_waves) < 128:
             k_splits //= 2
         sums = count = None
@@ -480,18 +480,24 @@ class HipKernels:
         return NormOwed(x_out, ssq_out, N, eps)
 
     @staticmethod
-    def _addnorm_splits(tiles, K):
-        """Workgroups that share one tile's K in ``linear_add_norm``. Measured on an MI355X at
-        the output and down projections of 4B-, 8B- and 32B-sized layers (tiles 160, 256, 320;
-        K 4,096 to 25,600; 1, 8 and 16 rows): meeting in memory costs about 2 us, so K is split
-        only where a tile per workgroup leaves the GPU unevenly filled (the tiles are no
-        multiple of its 256 compute units) and every wave keeps some 300 elements of K."""
-        if tiles % 256 == 0:
-            return 1
-        splits = 4
-        while splits > 1 and K // (splits * 8) < 300:
-            splits //= 2
-        return splits
+    def _addnorm_splits(tiles, K, M):
+        """Workgroups that share one tile's K in ``linear_add_norm``: 1, 2 or 4, whichever gives
+        the busiest of the GPU's 256 compute units the least to stream, with the meeting in
+        memory priced at some 3,000 elements of K (less at more rows, where streaming is
+        slower); every wave keeps some 300 elements. Measured on an MI355X at the output and
+        down projections of 4B-, 8B- and 32B-sized layers (tiles 160, 256, 320; K 4,096 to
+        25,600): 160 tiles of K = 9,728 take 12.3 us whole and 13.8 us in four parts at one row,
+        15.6 and 15.3 us at 8 rows, 19.8 and 17.8 us at 16; 320 tiles of K = 25,600 take 77 us
+        whole and 56 us in four parts at 8 rows."""
+        best, best_cost = 1, None
+        for splits in (1, 2, 4):
+            if splits > 1 and K // (splits * 8) < 300:
+                continue
+            rounds = -(-tiles * splits // 256)
+            cost = rounds * K / splits + (3000 * 8 / max(M, 8) if splits > 1 else 0)
+            if best_cost is None or cost < best_cost:
+                best, best_cost = splits, cost
+        return best
 
     # -- matrix products ------------------------------------------------------------------------
     def library_tuning(self, on: bool) -> None:
