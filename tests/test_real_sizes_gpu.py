@@ -42,7 +42,7 @@ def close(got, want, dtype, what):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_whole_prompt_then_captured_decode(wide, dtype):
-    """A 300-token prompt: most of it in one step, then its last 32 tokens one by one
+    """A 300-token prompt: most of it in two steps, then its last 32 tokens one by one
     through captured graphs (one row: the skinny products with K splits, the SwiGLU epilogue,
     the float32-output head of 151,936 rows, decode attention with key splits)."""
     from socrates_amd.engine import StepEntry
@@ -54,8 +54,13 @@ def test_whole_prompt_then_captured_decode(wide, dtype):
     runner = make_runner(folder, HipKernels(dtype, DEV), max_rows=2, max_len=512, block_size=16)
     runner.enable_graphs(2)
     row = runner.cache.open_row()
-    got = runner.step([StepEntry(row, prompt[:268], head_rows)]).float().cpu()
-    close(got, want[:len(head_rows)], dtype, "the prompt's first 268 tokens in one step")
+    # 218 tokens in one step, then a portion of 50: in bfloat16 the two projections into the
+    # residual sum of that step split K over sweeping workgroups (17 to 64 rows)
+    first = [r for r in head_rows if r < 218]
+    got = runner.step([StepEntry(row, prompt[:218], first)]).float().cpu()
+    close(got, want[:len(first)], dtype, "the prompt's first 218 tokens in one step")
+    got = runner.step([StepEntry(row, prompt[218:268], [r - 218 for r in head_rows[len(first):]])]).float().cpu()
+    close(got, want[len(first):len(head_rows)], dtype, "the next 50 tokens in one step")
     for t in range(268, 300):
         logits = runner.step([StepEntry(row, prompt[t:t + 1], [0])]).float().cpu()
         close(logits[0], want[len(head_rows) + t - 268], dtype, f"decoded token at position {t}")
