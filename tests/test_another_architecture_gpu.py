@@ -1,0 +1,148 @@
+"""Another architecture, added from this file alone: a configuration class with keys of its
+own, a plan whose layers differ (one with a window, feed-forwards of different sizes, tensor
+names of its own, an untied head), registered under its name. From there on everything is
+the framework's: the random-weights folder, the loader, the cache groups (the windowed layer
+gets pages of its own and gives them back), the step function with captured decode steps,
+and generation through ``Engine``. The oracle is put together from the plain implementation's
+functions, layer by layer, over whole sequences."""
+
+import json
+from dataclasses import dataclass
+from typing import Tuple
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from helpers import make_runner, random_prompts
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+# the tolerances and the weights' scale of the replay tests
+TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    """config.json of the toy: ``windows[i]`` 0 means that layer i sees every key."""
+    vocab: int
+    width: int
+    heads: int
+    kv_heads: int
+    head_size: int
+    ff_sizes: Tuple[int, ...]
+    windows: Tuple[int, ...]
+    eps: float
+    theta: float
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d["vocab"], d["width"], d["heads"], d["kv_heads"], d["head_size"], tuple(d["ff_sizes"]),
+                   tuple(d["windows"]), float(d["eps"]), float(d["theta"]))
+
+    def to_dict(self):
+        return dict(architectures=["ToyHybridLM"], vocab=self.vocab, width=self.width, heads=self.heads,
+                    kv_heads=self.kv_heads, head_size=self.head_size, ff_sizes=list(self.ff_sizes),
+                    windows=list(self.windows), eps=self.eps, theta=self.theta)
+
+    def plan(self):
+        from socrates_amd.config.specs import (AttentionSpec, BlockSpec, ModelPlan, RMSNormSpec, RopeSpec,
+                                               SwiGLUSpec, default_order)
+        norm = RMSNormSpec(self.width, self.eps)
+        layers = tuple(
+            BlockSpec(mixer=AttentionSpec(hidden=self.width, n_heads=self.heads, n_kv_heads=self.kv_heads,
+                                          head_dim=self.head_size, scale=self.head_size ** -0.5,
+                                          qk_norm=RMSNormSpec(self.head_size, self.eps),
+                                          position=RopeSpec(self.head_size, self.theta), window=w or None),
+                      ffn=SwiGLUSpec(self.width, ff), norm1=norm, norm2=norm, prefix=f"blocks.{i}.",
+                      names=(("norm1", "ln_a"), ("mixer", "attn"), ("norm2", "ln_b"), ("ffn", "ff")))
+            for i, (ff, w) in enumerate(zip(self.ff_sizes, self.windows)))
+        return ModelPlan(architecture="ToyHybridLM", vocab_size=self.vocab, hidden=self.width, layers=layers,
+                         order=default_order(len(layers)), final_norm=norm, embedding_name="tok.weight",
+                         final_norm_prefix="ln_out", head_name="out.weight")
+
+
+TOY = HybridConfig(vocab=301, width=96, heads=6, kv_heads=2, head_size=32, ff_sizes=(136, 72, 200),
+                   windows=(0, 7, 0), eps=3e-6, theta=5e4)
+
+
+def oracle(cfg, w, ids, rows):
+    """Logits at ``rows`` of the whole sequence, from the plain implementation's parts."""
+    ids = torch.as_tensor(ids, dtype=torch.long)
+    positions = torch.arange(len(ids))
+    part = dict(num_attention_heads=cfg["heads"], num_key_value_heads=cfg["kv_heads"], head_dim=cfg["head_size"],
+                rms_norm_eps=cfg["eps"], rope_theta=cfg["theta"])
+    x = w["tok.weight"][ids]
+    for i, window in enumerate(cfg["windows"]):
+        p = f"blocks.{i}."
+        x = x + plain.attention_layer(plain.rms_norm(x, w[p + "ln_a.weight"], cfg["eps"]), w, p + "attn.", part,
+                                      positions, window or None)
+        x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "ln_b.weight"], cfg["eps"]), w, p + "ff.")
+    x = plain.rms_norm(x[torch.as_tensor(rows)], w["ln_out.weight"], cfg["eps"])
+    return x @ w["out.weight"].T
+
+
+@pytest.fixture(scope="module")
+def toy_folder(tmp_path_factory):
+    from socrates_amd.config import load_config, register_architecture
+    from socrates_amd.weights import write_random_model
+    register_architecture("ToyHybridLM", HybridConfig)
+    folder = write_random_model(tmp_path_factory.mktemp("hybrid") / "m", TOY, 9, dtype=torch.bfloat16,
+                                std=0.05, gain_std=0.1)
+    assert json.loads((folder / "config.json").read_text())["windows"] == [0, 7, 0]
+    assert load_config(folder) == TOY
+    cfg, w = plain.read_folder(folder)
+    return folder, cfg, w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_portions_and_captured_decode_of_the_new_architecture(toy_folder, dtype):
+    """Two requests: prompts in portions of changing size beside each other, then decoded
+    tokens one by one through captured graphs; every logit against the oracle. The windowed
+    layer is a cache group of its own whose pages come back while the request is alive."""
+    from socrates_amd.engine import StepEntry
+    from socrates_amd.kernels import HipKernels
+    folder, cfg, w = toy_folder
+    a, b = random_prompts([45, 30], cfg["vocab"], seed=3)
+    runner = make_runner(folder, HipKernels(dtype, DEV), max_rows=2, max_len=64, block_size=4)
+    groups = runner.cache.groups
+    assert sorted(g.need.window or 0 for g in groups) == [0, 7]
+    assert [len(g.pools) for g in groups if not g.need.window] == [2]       # the two layers that see every key share a group
+    runner.enable_graphs(2)
+    ra, rb = runner.cache.open_row(), runner.cache.open_row()
+    want_a, want_b = oracle(cfg, w, a, list(range(45))), oracle(cfg, w, b, list(range(30)))
+
+    def check(got, want, what):
+        tol = TOL[dtype]
+        torch.testing.assert_close(got.float().cpu(), want, msg=lambda m: f"{what}: {m}", **tol)
+
+    cuts_a, cuts_b = [(0, 17), (17, 19), (19, 33)], [(0, 2), (2, 20), (20, 22)]
+    for (a0, a1), (b0, b1) in zip(cuts_a, cuts_b):
+        got = runner.step([StepEntry(ra, a[a0:a1], list(range(a1 - a0))), StepEntry(rb, b[b0:b1], list(range(b1 - b0)))])
+        check(got[:a1 - a0], want_a[a0:a1], f"a[{a0}:{a1}]")
+        check(got[a1 - a0:], want_b[b0:b1], f"b[{b0}:{b1}]")
+    windowed = next(g for g in groups if g.need.window)
+    full = next(g for g in groups if not g.need.window)
+    assert len(windowed.held_by(ra)) < len(full.held_by(ra))           # pages behind the window went back
+    for t in range(8):
+        got = runner.step([StepEntry(ra, [a[33 + t]], [0]), StepEntry(rb, [b[22 + t]], [0])])
+        check(got[0], want_a[33 + t], f"a, decoded at {33 + t}")
+        check(got[1], want_b[22 + t], f"b, decoded at {22 + t}")
+    assert runner._graphs                                               # the decode steps were captured ones
+    runner.cache.close_row(ra)
+    runner.cache.close_row(rb)
+    assert not runner.cache.open_rows
+
+
+def test_greedy_generation_of_the_new_architecture_through_the_engine(toy_folder):
+    """``Engine(folder)`` finds the architecture by its name; float32 tokens are the oracle's."""
+    from socrates_amd.engine import Engine
+    folder, cfg, w = toy_folder
+    prompts = random_prompts([11, 4, 19], cfg["vocab"], seed=4)
+    engine = Engine(str(folder), device=DEV, dtype=torch.float32, max_batch=4, max_len=64, block_size=4)
+    got = engine.generate(prompts, max_new_tokens=9)
+    for prompt, out in zip(prompts, got):
+        seq = list(prompt)
+        for _ in range(9):
+            seq.append(int(oracle(cfg, w, seq, [len(seq) - 1])[0].argmax()))
+        assert out == seq[len(prompt):]
