@@ -1,6 +1,7 @@
 """Another architecture, added from this file alone: a configuration class with keys of its
-own, a plan whose layers differ (one with a window, feed-forwards of different sizes, tensor
-names of its own, an untied head), registered under its name. From there on everything is
+own, a plan whose layers differ (one with a window, feed-forwards of different sizes, one layer
+in an arrangement of its own that this file registers, tensor names of its own, an untied
+head), registered under its name. From there on everything is
 the framework's: the random-weights folder, the loader, the cache groups (the windowed layer
 gets pages of its own and gives them back), the step function with captured decode steps,
 and generation through ``Engine``. The oracle is put together from the plain implementation's
@@ -22,9 +23,28 @@ DEV = "cuda:0"
 TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
 
 
+class ParallelBlock:
+    """An arrangement from outside: y = x + mixer(norm1(x)) + ffn(norm1(x)). Like every block it
+    gets the float32 residual stream and the previous block's output not yet added to it, and
+    returns its own output un-added; the second norm of the spec is not used."""
+
+    def __init__(self, spec, weights, ops):
+        from socrates_amd.parts.registry import build_part, tensors_of
+
+        def sub(role):
+            part = getattr(spec, role)
+            return build_part(part, {name: weights[f"{spec.name_of(role)}.{name}"] for name in tensors_of(part)}, ops)
+        self.norm1, self.mixer, self.ffn = sub("norm1"), sub("mixer"), sub("ffn")
+
+    def forward(self, residual, pending, ctx, slot, write=True):
+        h = self.norm1.add_norm(residual, pending)
+        return self.mixer.forward(h, ctx, slot, write) + self.ffn.forward(h, ctx)
+
+
 @dataclass(frozen=True)
 class HybridConfig:
-    """config.json of the toy: ``windows[i]`` 0 means that layer i sees every key."""
+    """config.json of the toy: ``windows[i]`` 0 means that layer i sees every key; layers
+    listed in ``parallel`` run mixer and feed-forward side by side."""
     vocab: int
     width: int
     heads: int
@@ -32,18 +52,19 @@ class HybridConfig:
     head_size: int
     ff_sizes: Tuple[int, ...]
     windows: Tuple[int, ...]
+    parallel: Tuple[int, ...]
     eps: float
     theta: float
 
     @classmethod
     def from_dict(cls, d):
         return cls(d["vocab"], d["width"], d["heads"], d["kv_heads"], d["head_size"], tuple(d["ff_sizes"]),
-                   tuple(d["windows"]), float(d["eps"]), float(d["theta"]))
+                   tuple(d["windows"]), tuple(d["parallel"]), float(d["eps"]), float(d["theta"]))
 
     def to_dict(self):
         return dict(architectures=["ToyHybridLM"], vocab=self.vocab, width=self.width, heads=self.heads,
                     kv_heads=self.kv_heads, head_size=self.head_size, ff_sizes=list(self.ff_sizes),
-                    windows=list(self.windows), eps=self.eps, theta=self.theta)
+                    windows=list(self.windows), parallel=list(self.parallel), eps=self.eps, theta=self.theta)
 
     def plan(self):
         from socrates_amd.config.specs import (AttentionSpec, BlockSpec, ModelPlan, RMSNormSpec, RopeSpec,
@@ -55,7 +76,8 @@ class HybridConfig:
                                           qk_norm=RMSNormSpec(self.head_size, self.eps),
                                           position=RopeSpec(self.head_size, self.theta), window=w or None),
                       ffn=SwiGLUSpec(self.width, ff), norm1=norm, norm2=norm, prefix=f"blocks.{i}.",
-                      names=(("norm1", "ln_a"), ("mixer", "attn"), ("norm2", "ln_b"), ("ffn", "ff")))
+                      names=(("norm1", "ln_a"), ("mixer", "attn"), ("norm2", "ln_b"), ("ffn", "ff")),
+                      arrangement="parallel" if i in self.parallel else "prenorm")
             for i, (ff, w) in enumerate(zip(self.ff_sizes, self.windows)))
         return ModelPlan(architecture="ToyHybridLM", vocab_size=self.vocab, hidden=self.width, layers=layers,
                          order=default_order(len(layers)), final_norm=norm, embedding_name="tok.weight",
@@ -63,7 +85,7 @@ class HybridConfig:
 
 
 TOY = HybridConfig(vocab=301, width=96, heads=6, kv_heads=2, head_size=32, ff_sizes=(136, 72, 200),
-                   windows=(0, 7, 0), eps=3e-6, theta=5e4)
+                   windows=(0, 7, 0), parallel=(2,), eps=3e-6, theta=5e4)
 
 
 def oracle(cfg, w, ids, rows):
@@ -75,9 +97,11 @@ def oracle(cfg, w, ids, rows):
     x = w["tok.weight"][ids]
     for i, window in enumerate(cfg["windows"]):
         p = f"blocks.{i}."
-        x = x + plain.attention_layer(plain.rms_norm(x, w[p + "ln_a.weight"], cfg["eps"]), w, p + "attn.", part,
-                                      positions, window or None)
-        x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "ln_b.weight"], cfg["eps"]), w, p + "ff.")
+        h = plain.rms_norm(x, w[p + "ln_a.weight"], cfg["eps"])
+        x = x + plain.attention_layer(h, w, p + "attn.", part, positions, window or None)
+        if i not in cfg["parallel"]:
+            h = plain.rms_norm(x, w[p + "ln_b.weight"], cfg["eps"])
+        x = x + plain.swiglu_mlp(h, w, p + "ff.")
     x = plain.rms_norm(x[torch.as_tensor(rows)], w["ln_out.weight"], cfg["eps"])
     return x @ w["out.weight"].T
 
@@ -85,8 +109,10 @@ def oracle(cfg, w, ids, rows):
 @pytest.fixture(scope="module")
 def toy_folder(tmp_path_factory):
     from socrates_amd.config import load_config, register_architecture
+    from socrates_amd.parts.block import register_arrangement
     from socrates_amd.weights import write_random_model
     register_architecture("ToyHybridLM", HybridConfig)
+    register_arrangement("parallel", ParallelBlock)
     folder = write_random_model(tmp_path_factory.mktemp("hybrid") / "m", TOY, 9, dtype=torch.bfloat16,
                                 std=0.05, gain_std=0.1)
     assert json.loads((folder / "config.json").read_text())["windows"] == [0, 7, 0]
