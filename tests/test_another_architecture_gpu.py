@@ -1,7 +1,7 @@
 """Another architecture, added from this file alone: a configuration class with keys of its
 own, a plan whose layers differ (one with a window, feed-forwards of different sizes, one layer
-in an arrangement of its own that this file registers, tensor names of its own, an untied
-head), registered under its name. From there on everything is
+in an arrangement of its own and a norm of its own that this file registers, tensor names of
+its own, an untied head), registered under its name. From there on everything is
 the framework's: the random-weights folder, the loader, the cache groups (the windowed layer
 gets pages of its own and gives them back), the step function with captured decode steps,
 and generation through ``Engine``. The oracle is put together from the plain implementation's
@@ -38,7 +38,45 @@ class ParallelBlock:
 
     def forward(self, residual, pending, ctx, slot, write=True):
         h = self.norm1.add_norm(residual, pending)
-        return self.mixer.forward(h, ctx, slot, write) + self.ffn.forward(h, ctx)
+        both = (self.mixer.forward(h, ctx, slot, write), self.ffn.forward(h, ctx))
+        # either may come as float32 partial sums [S, N, d]; so does what this block returns,
+        # and the norm that runs next adds them to the residual stream in order
+        return torch.cat([t if t.dim() == 3 else t.float().unsqueeze(0) for t in both])
+
+
+@dataclass(frozen=True)
+class CenterNormSpec:
+    """y = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias over the last ``dim`` elements."""
+    dim: int
+    eps: float
+
+
+class CenterNorm:
+    """A norm from outside, written with library routines: it has no ``fusable``, so the blocks
+    around it run product, sum and norm one after the other."""
+
+    @staticmethod
+    def tensors(spec):
+        from socrates_amd.parts.registry import TensorDecl
+        return {"weight": TensorDecl((spec.dim,), "vector"), "bias": TensorDecl((spec.dim,), "vector")}
+
+    def __init__(self, spec, tensors, ops):
+        self.spec, self.ops, self.weight, self.bias = spec, ops, tensors["weight"], tensors["bias"]
+
+    def add_norm(self, residual, delta, rows=None):
+        if delta is not None:
+            delta = delta.sum(0) if delta.dim() == 3 else delta.float()
+        if rows is None:
+            if delta is not None:
+                residual += delta
+            h = residual
+        else:
+            h = residual[rows.long()] + (delta[rows.long()] if delta is not None else 0)
+        return self(h)
+
+    def __call__(self, x):
+        y = torch.nn.functional.layer_norm(x.float(), (self.spec.dim,), self.weight, self.bias, self.spec.eps)
+        return y.to(self.ops.dtype)
 
 
 @dataclass(frozen=True)
@@ -69,18 +107,19 @@ class HybridConfig:
     def plan(self):
         from socrates_amd.config.specs import (AttentionSpec, BlockSpec, ModelPlan, RMSNormSpec, RopeSpec,
                                                SwiGLUSpec, default_order)
-        norm = RMSNormSpec(self.width, self.eps)
+        norm, centred = RMSNormSpec(self.width, self.eps), CenterNormSpec(self.width, self.eps)
         layers = tuple(
             BlockSpec(mixer=AttentionSpec(hidden=self.width, n_heads=self.heads, n_kv_heads=self.kv_heads,
                                           head_dim=self.head_size, scale=self.head_size ** -0.5,
                                           qk_norm=RMSNormSpec(self.head_size, self.eps),
                                           position=RopeSpec(self.head_size, self.theta), window=w or None),
-                      ffn=SwiGLUSpec(self.width, ff), norm1=norm, norm2=norm, prefix=f"blocks.{i}.",
+                      ffn=SwiGLUSpec(self.width, ff), norm1=centred if i in self.parallel else norm, norm2=norm,
+                      prefix=f"blocks.{i}.",
                       names=(("norm1", "ln_a"), ("mixer", "attn"), ("norm2", "ln_b"), ("ffn", "ff")),
                       arrangement="parallel" if i in self.parallel else "prenorm")
             for i, (ff, w) in enumerate(zip(self.ff_sizes, self.windows)))
         return ModelPlan(architecture="ToyHybridLM", vocab_size=self.vocab, hidden=self.width, layers=layers,
-                         order=default_order(len(layers)), final_norm=norm, embedding_name="tok.weight",
+                         order=default_order(len(layers)), final_norm=centred, embedding_name="tok.weight",
                          final_norm_prefix="ln_out", head_name="out.weight")
 
 
@@ -97,22 +136,28 @@ def oracle(cfg, w, ids, rows):
     x = w["tok.weight"][ids]
     for i, window in enumerate(cfg["windows"]):
         p = f"blocks.{i}."
-        h = plain.rms_norm(x, w[p + "ln_a.weight"], cfg["eps"])
+        if i in cfg["parallel"]:
+            h = torch.nn.functional.layer_norm(x, (cfg["width"],), w[p + "ln_a.weight"], w[p + "ln_a.bias"], cfg["eps"])
+        else:
+            h = plain.rms_norm(x, w[p + "ln_a.weight"], cfg["eps"])
         x = x + plain.attention_layer(h, w, p + "attn.", part, positions, window or None)
         if i not in cfg["parallel"]:
             h = plain.rms_norm(x, w[p + "ln_b.weight"], cfg["eps"])
         x = x + plain.swiglu_mlp(h, w, p + "ff.")
-    x = plain.rms_norm(x[torch.as_tensor(rows)], w["ln_out.weight"], cfg["eps"])
+    x = torch.nn.functional.layer_norm(x[torch.as_tensor(rows)], (cfg["width"],), w["ln_out.weight"],
+                                       w["ln_out.bias"], cfg["eps"])
     return x @ w["out.weight"].T
 
 
 @pytest.fixture(scope="module")
 def toy_folder(tmp_path_factory):
     from socrates_amd.config import load_config, register_architecture
+    from socrates_amd.parts import register_part
     from socrates_amd.parts.block import register_arrangement
     from socrates_amd.weights import write_random_model
     register_architecture("ToyHybridLM", HybridConfig)
     register_arrangement("parallel", ParallelBlock)
+    register_part(CenterNormSpec, CenterNorm)
     folder = write_random_model(tmp_path_factory.mktemp("hybrid") / "m", TOY, 9, dtype=torch.bfloat16,
                                 std=0.05, gain_std=0.1)
     assert json.loads((folder / "config.json").read_text())["windows"] == [0, 7, 0]
