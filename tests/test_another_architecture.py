@@ -17,8 +17,11 @@ import torch
 import plain_qwen3 as plain
 from helpers import make_runner, random_prompts
 
-pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+# the torch stand-in for the kernels on the CPU, the HIP kernels in both precisions on the GPU
+KINDS = [pytest.param("torch", torch.float32, id="cpu-fp32"),
+         pytest.param("hip", torch.float32, id="gpu-fp32", marks=pytest.mark.gpu),
+         pytest.param("hip", torch.bfloat16, id="gpu-bf16", marks=pytest.mark.gpu)]
 # the tolerances and the weights' scale of the replay tests
 TOL = {torch.float32: dict(atol=1e-4, rtol=1e-4), torch.bfloat16: dict(atol=6e-2, rtol=5e-2)}
 
@@ -166,20 +169,27 @@ def toy_folder(tmp_path_factory):
     return folder, cfg, w
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-def test_portions_and_captured_decode_of_the_new_architecture(toy_folder, dtype):
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_portions_and_decode_of_the_new_architecture(toy_folder, kind, dtype):
     """Two requests: prompts in portions of changing size beside each other, then decoded
-    tokens one by one through captured graphs; every logit against the oracle. The windowed
-    layer is a cache group of its own whose pages come back while the request is alive."""
+    tokens one by one (through captured graphs on the GPU); every logit against the oracle.
+    The windowed layer is a cache group of its own whose pages come back while the request
+    is alive."""
     from socrates_amd.engine import StepEntry
-    from socrates_amd.kernels import HipKernels
     folder, cfg, w = toy_folder
+    if kind == "hip":
+        from socrates_amd.kernels import HipKernels
+        ops = HipKernels(dtype, DEV)
+    else:
+        from torch_kernels import TorchKernels
+        ops = TorchKernels(dtype, "cpu")
     a, b = random_prompts([45, 30], cfg["vocab"], seed=3)
-    runner = make_runner(folder, HipKernels(dtype, DEV), max_rows=2, max_len=64, block_size=4)
+    runner = make_runner(folder, ops, max_rows=2, max_len=64, block_size=4)
     groups = runner.cache.groups
     assert sorted(g.need.window or 0 for g in groups) == [0, 7]
     assert [len(g.pools) for g in groups if not g.need.window] == [2]       # the two layers that see every key share a group
-    runner.enable_graphs(2)
+    if kind == "hip":
+        runner.enable_graphs(2)
     ra, rb = runner.cache.open_row(), runner.cache.open_row()
     want_a, want_b = oracle(cfg, w, a, list(range(45))), oracle(cfg, w, b, list(range(30)))
 
@@ -199,12 +209,13 @@ def test_portions_and_captured_decode_of_the_new_architecture(toy_folder, dtype)
         got = runner.step([StepEntry(ra, [a[33 + t]], [0]), StepEntry(rb, [b[22 + t]], [0])])
         check(got[0], want_a[33 + t], f"a, decoded at {33 + t}")
         check(got[1], want_b[22 + t], f"b, decoded at {22 + t}")
-    assert runner._graphs                                               # the decode steps were captured ones
+    assert kind != "hip" or runner._graphs                              # the decode steps were captured ones
     runner.cache.close_row(ra)
     runner.cache.close_row(rb)
     assert not runner.cache.open_rows
 
 
+@pytest.mark.gpu
 def test_greedy_generation_of_the_new_architecture_through_the_engine(toy_folder):
     """``Engine(folder)`` finds the architecture by its name; float32 tokens are the oracle's."""
     from socrates_amd.engine import Engine
