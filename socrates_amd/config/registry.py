@@ -25,7 +25,27 @@ def known_architectures():
     return sorted(_ARCHITECTURES)
 
 
+_plugins_loaded = False
+
+
+def _load_plugins() -> None:
+    """Import the modules that SOCRATES_AMD_PLUGINS names, once."""
+    global _plugins_loaded
+    if _plugins_loaded:
+        return
+    _plugins_loaded = True
+    import importlib
+    import os
+    for module in filter(None, (m.strip() for m in os.environ.get("SOCRATES_AMD_PLUGINS", "").split(","))):
+        try:
+            importlib.import_module(module)
+        except ImportError as e:
+            raise ConfigError(f"SOCRATES_AMD_PLUGINS names {module!r}, which cannot be imported: {e}") from e
+
+
 def config_class_for(name: str):
+    if name not in _ARCHITECTURES:
+        _load_plugins()
     try:
         return _ARCHITECTURES[name]
     except KeyError:

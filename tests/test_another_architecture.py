@@ -152,15 +152,21 @@ def oracle(cfg, w, ids, rows):
     return x @ w["out.weight"].T
 
 
-@pytest.fixture(scope="module")
-def toy_folder(tmp_path_factory):
-    from socrates_amd.config import load_config, register_architecture
+def register():
+    """All that the framework has to be told."""
+    from socrates_amd.config import register_architecture
     from socrates_amd.parts import register_part
     from socrates_amd.parts.block import register_arrangement
-    from socrates_amd.weights import write_random_model
     register_architecture("ToyHybridLM", HybridConfig)
     register_arrangement("parallel", ParallelBlock)
     register_part(CenterNormSpec, CenterNorm)
+
+
+@pytest.fixture(scope="module")
+def toy_folder(tmp_path_factory):
+    from socrates_amd.config import load_config
+    from socrates_amd.weights import write_random_model
+    register()
     folder = write_random_model(tmp_path_factory.mktemp("hybrid") / "m", TOY, 9, dtype=torch.bfloat16,
                                 std=0.05, gain_std=0.1)
     assert json.loads((folder / "config.json").read_text())["windows"] == [0, 7, 0]
@@ -228,3 +234,35 @@ def test_greedy_generation_of_the_new_architecture_through_the_engine(toy_folder
         for _ in range(9):
             seq.append(int(oracle(cfg, w, seq, [len(seq) - 1])[0].argmax()))
         assert out == seq[len(prompt):]
+
+
+@pytest.mark.gpu
+def test_the_replay_program_serves_it_as_a_plug_in(toy_folder, tmp_path):
+    """``bin/trace_run`` in a process of its own knows nothing of the toy until the module
+    named in SOCRATES_AMD_PLUGINS registers it; then the folder's config.json chooses it as
+    it chooses any architecture, and the logits are the oracle's."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+    import numpy as np
+    folder, cfg, w = toy_folder
+    root = Path(__file__).resolve().parent.parent
+    (tmp_path / "toy_plugin.py").write_text("import test_another_architecture\ntest_another_architecture.register()\n")
+    (prompt,) = random_prompts([21], cfg["vocab"], seed=6)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": prompt[:13], "want": [0, 12]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": prompt[13:], "want": list(range(8))}], "end": ["a"]}]
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join([str(tmp_path), str(Path(__file__).resolve().parent),
+                                                       os.environ.get("PYTHONPATH", "")]))
+    cmd = [sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32",
+           "--out", str(tmp_path / "out"), "--max-tokens", "64"]
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    unknown = subprocess.run(cmd, input=text, capture_output=True, text=True, env=env, timeout=300)
+    assert unknown.returncode != 0 and "unknown architecture 'ToyHybridLM'" in unknown.stderr
+    proc = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=300,
+                          env=dict(env, SOCRATES_AMD_PLUGINS="toy_plugin"))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1"]
+    want = oracle(cfg, w, prompt, [0, 12] + list(range(13, 21)))
+    got = np.concatenate([np.fromfile(tmp_path / "out" / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]) for i in (0, 1)])
+    torch.testing.assert_close(torch.from_numpy(got), want, **TOL[torch.float32])

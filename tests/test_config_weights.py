@@ -98,6 +98,27 @@ def test_registry(tmp_path):
     assert type(load_config(tmp_path)) is Other
 
 
+def test_plug_ins_named_in_the_environment(tmp_path, monkeypatch):
+    """A module named in SOCRATES_AMD_PLUGINS is imported when a name is looked up that the
+    registry does not know, and may register it; a module that cannot be imported is one
+    clear error."""
+    import socrates_amd.config.registry as registry
+    (tmp_path / "plug_a.py").write_text(
+        "from socrates_amd.config import Qwen3Config, register_architecture\n"
+        "class Plugged(Qwen3Config):\n    pass\n"
+        "register_architecture('PluggedLM', Plugged)\n")
+    (tmp_path / "config.json").write_text(json.dumps(dict(TINY_A["cfg"], architectures=["PluggedLM"])))
+    monkeypatch.syspath_prepend(str(tmp_path))
+    monkeypatch.setattr(registry, "_plugins_loaded", False)
+    monkeypatch.setenv("SOCRATES_AMD_PLUGINS", "no_such_module_anywhere")
+    with pytest.raises(ConfigError, match="no_such_module_anywhere.*cannot be imported"):
+        load_config(tmp_path)
+    monkeypatch.setattr(registry, "_plugins_loaded", False)
+    monkeypatch.setenv("SOCRATES_AMD_PLUGINS", " plug_a ,")
+    assert type(load_config(tmp_path)).__name__ == "Plugged"
+    registry._ARCHITECTURES.pop("PluggedLM")
+
+
 def test_presets_that_come_with_the_package():
     """Five configuration files: the two tiny test shapes and Qwen3-4B, -8B and -32B sizes.
     Parameter counts of the big ones are the published model sizes; the 4B file says what the
