@@ -15,7 +15,7 @@
 //                        optional SwiGLU epilogue.
 //  gemm_bf16_sweep_kernel the same product for at most 16 rows with one workgroup per compute
 //                        unit that keeps its slices of x in registers and walks over the
-//                        weight tiles (K up to 4,096).
+//                        weight tiles (K up to 5,120).
 //  gemm_bf16_sweep_parts_kernel 17 to 64 rows: K split over such workgroups, float32 partial
 //                        sums for a consumer that adds them.
 #include "common.h"
@@ -694,7 +694,7 @@ SOC_EXPORT int soc_gemm_bf16_skinny(const void* X, const void* W, void* C, float
 // kernel's time at 8 rows and a third at 16 (a build without the loads of x runs at the
 // one-row speed whatever M is). Here a product has at most one workgroup per compute unit,
 // of 16 waves that split K as before; a wave keeps its slices of x in registers for the
-// whole kernel (at most 8 steps of 32 k, so K up to 4,096), and the workgroup sweeps over
+// whole kernel (at most 8 steps of 32 k, or two halves of 5: K up to 5,120), and the workgroup sweeps over
 // weight tiles g, g + G, g + 2 G, ...: per tile a wave loads only weights, multiplies, and
 // leaves its sums in LDS, where the first four waves add them and do the epilogue while the
 // others go on. The weights of two tiles are on their way at any time, and x is read once per
@@ -715,7 +715,11 @@ struct SwPlan {
     int items;                      // weight tiles (tile pairs with SWIGLU)
 };
 
-template <typename TC, int MODE, int MAXS>
+// HALVES 2 (K from 4,097 to 16 x 2 x 5 x 32 = 5,120): a wave's share of K in two halves of at most
+// MAXS steps. Its slices of x for both stay in registers; the two buffers of weights hold the
+// two halves of one tile, each asked for anew (for the next tile) as soon as it is multiplied,
+// so a tile's worth of weights is on its way at any time, as with one half.
+template <typename TC, int MODE, int MAXS, int HALVES = 1>
 __global__ void __launch_bounds__(1024)
 gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C, int M,
                        int N, int K, SwPlan pl, SkNorm nm, int layout) {
@@ -746,36 +750,37 @@ gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, T
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(W), (short)0, (int)((size_t)N * K * 2), 0x00020000);
     // (the weights row by row or by tile, as in the skinny kernel)
     const int w_rs = w_tiled ? 32 : K, w_ss = w_tiled ? 512 : 32;
-    uint4 xr[MAXS];
-    uint32_t k_off[MAXS];                               // byte offset of the slice from its tile's row 0, or nowhere
+    uint4 xr[HALVES][MAXS];
+    uint32_t k_off[HALVES][MAXS];                       // byte offset of the slice from its tile's row 0, or nowhere
 #pragma unroll
-    for (int s = 0; s < MAXS; ++s) {
-        const int k = k_begin + 32 * s + lk;
-        k_off[s] = k < k_end ? (uint32_t)((((k_begin / 32 + s) * w_ss) + li * w_rs + lk) * 2) : SW_NOWHERE;
-        xr[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                    x_rsrc, k < k_end ? (uint32_t)((li * K + k) * 2) : SW_NOWHERE, 0, 0));
-    }
-    auto load_w = [&](uint4 (&wb)[MAXS], int q) {
+    for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) {
+            const int step = h * MAXS + s, k = k_begin + 32 * step + lk;
+            k_off[h][s] = k < k_end ? (uint32_t)((((k_begin / 32 + step) * w_ss) + li * w_rs + lk) * 2) : SW_NOWHERE;
+            xr[h][s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                           x_rsrc, k < k_end ? (uint32_t)((li * K + k) * 2) : SW_NOWHERE, 0, 0));
+        }
+    auto load_w = [&](uint4 (&wb)[MAXS], int q, int h = 0) {
         const bool live = q < n_sub;                    // the same for the whole workgroup
         // a tile starts at 16 K t either way; a weight row beyond N lies beyond the descriptor's end
         const uint32_t row = live ? (uint32_t)((size_t)tile_of(live ? q : 0) * 16 * K * 2) : 0u;
 #pragma unroll
         for (int s = 0; s < MAXS; ++s)
             wb[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                        w_rsrc, live && k_off[s] != SW_NOWHERE ? row + k_off[s] : SW_NOWHERE, 0, 0));
+                        w_rsrc, live && k_off[h][s] != SW_NOWHERE ? row + k_off[h][s] : SW_NOWHERE, 0, 0));
     };
-    auto compute = [&](const uint4 (&wb)[MAXS]) {
-        f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const uint4 (&wb)[MAXS], int h = 0, f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f}) {
 #pragma unroll
         for (int s = 0; s < MAXS; ++s)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wb[s]),
-                                                          __builtin_bit_cast(bf16x8, xr[s]), acc, 0, 0, 0);
+                                                          __builtin_bit_cast(bf16x8, xr[h][s]), acc, 0, 0, 0);
         return acc;
     };
 
     uint4 wa[MAXS], wb2[MAXS];
     load_w(wa, 0);
-    load_w(wb2, 1);
+    load_w(wb2, HALVES == 1 ? 1 : 0, HALVES - 1);
     if constexpr (SCALED) {
         // the norm's factor of every row, once per workgroup, while the first loads are on their way
         const int stride = sk_ssq_stride(nm.ssq_tiles);
@@ -820,23 +825,39 @@ gemm_bf16_sweep_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, T
     // parity: the reducers read one half while the next tile's sums are written to the other,
     // and one barrier per tile orders both. Past the end of the sweep a round loads zeros
     // from nowhere and has no epilogue, but the barrier all the same.
-    for (int q = 0; q < n_sub; q += 2) {
-        leave(compute(wa), 0);
-        load_w(wa, q + 2);
-        finish(q, 0);
-        leave(compute(wb2), 1);
-        load_w(wb2, q + 3);
-        finish(q + 1, 1);
+    if constexpr (HALVES == 1) {
+        for (int q = 0; q < n_sub; q += 2) {
+            leave(compute(wa), 0);
+            load_w(wa, q + 2);
+            finish(q, 0);
+            leave(compute(wb2), 1);
+            load_w(wb2, q + 3);
+            finish(q + 1, 1);
+        }
+    } else {
+        // `wa` holds the first half of a tile's K, `wb2` the second
+        auto one = [&](int q, int p) {
+            f32x4 acc = compute(wa, 0);
+            load_w(wa, q + 1, 0);
+            acc = compute(wb2, 1, acc);
+            load_w(wb2, q + 1, 1);
+            leave(acc, p);
+            finish(q, p);
+        };
+        for (int q = 0; q < n_sub; q += 2) {
+            one(q, 0);
+            one(q + 1, 1);
+        }
     }
 }
 
 // Shape of a sweep for an [M <= 16] x [N, K] product: waves per workgroup and workgroups; 0
-// if the sweep form does not apply (K longer than 16 waves x 256). The tiles (pairs) are
+// if the sweep form does not apply (K longer than 16 waves x 320). The tiles (pairs) are
 // shared out so that the GPU's 256 compute units get at most one workgroup each, with equal
 // numbers of tiles as far as that goes.
 SOC_EXPORT int soc_gemm_sweep_plan(int N, int K, int swiglu, int* n_waves, int* workgroups) {
     const int nw = 16;
-    if (K > nw * 256) return 0;
+    if (K > nw * 320) return 0;                         // 8 steps of 32 per wave, or two halves of 5
     const int items = swiglu ? N / 32 : (N + 15) / 16;
     if (items < 1) return 0;
     const int per_wg = (items + 255) / 256;
@@ -847,7 +868,7 @@ SOC_EXPORT int soc_gemm_sweep_plan(int N, int K, int swiglu, int* n_waves, int* 
 
 // mode: SK_SWIGLU (C [M, N / 2], N a multiple of 32) or 0 (C [M, N] in c_dtype), each with or
 // without SK_SCALED (ssq_in, ssq_tiles, norm_dim, eps; bfloat16 output). K / n_waves rounded
-// up to 32 must not exceed 256. The matrices lie below 4 GiB.
+// up to 32 must not exceed 320. The matrices lie below 4 GiB.
 SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
                                    int mode, int n_waves, int workgroups, const float* ssq_in, int ssq_tiles,
                                    int norm_dim, float eps, int layout, hipStream_t stream) {
@@ -865,7 +886,7 @@ SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M,
     if (c_dtype == 0 && mode != 0) return (int)hipErrorInvalidValue;            // float32 output: the plain form only
     SwPlan pl;
     pl.k_per_wave = ((K + n_waves - 1) / n_waves + 31) / 32 * 32;
-    if (pl.k_per_wave > 256) return (int)hipErrorInvalidValue;
+    if (pl.k_per_wave > 320) return (int)hipErrorInvalidValue;
     pl.items = swiglu ? N / 32 : (N + 15) / 16;
     SkNorm nm{};
     nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
@@ -877,7 +898,9 @@ SOC_EXPORT int soc_gemm_bf16_sweep(const void* X, const void* W, void* C, int M,
 #define SOC_SW_STEPS(TC_, MODE_)                                                           \
     do {                                                                                   \
         if (steps <= 2) SOC_SW(TC_, MODE_, 2); else if (steps <= 4) SOC_SW(TC_, MODE_, 4); \
-        else if (steps <= 5) SOC_SW(TC_, MODE_, 5); else SOC_SW(TC_, MODE_, 8);            \
+        else if (steps <= 5) SOC_SW(TC_, MODE_, 5); else if (steps <= 8) SOC_SW(TC_, MODE_, 8); \
+        else hipLaunchKernelGGL((gemm_bf16_sweep_kernel<TC_, MODE_, 5, 2>), grid, block, 0, stream, (const bf16*)X, \
+                                (const bf16*)W, (TC_*)C, M, N, K, pl, nm, layout);         \
     } while (0)
     if (c_dtype == 0) { SOC_SW_STEPS(float, 0); return soc_last_error(); }
     switch (mode) {

@@ -218,14 +218,16 @@ def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
 
 
 @pytest.mark.parametrize("M,d,K", [(1, 64, 64), (8, 2560, 4096), (16, 72, 200), (5, 104, 4088), (3, 4096, 96),
-                                   (11, 2560, 2568), (7, 330, 1000), (16, 6144, 2560), (4, 48, 8)])
+                                   (11, 2560, 2568), (7, 330, 1000), (16, 6144, 2560), (4, 48, 8),
+                                   (8, 5120, 5120), (16, 208, 4616), (1, 1024, 4104)])
 def test_sweep_form_of_the_skinny_products(kernel_sets, M, d, K):
     """The products of at most 16 rows in their sweep form (a workgroup keeps its slices of x
     in registers and walks over the weight tiles), forced on at every size: plain, with
     float32 output, and the two kinds of product that consume rows owed a norm (plain and
     gate / up with the activation), against float64 and against the form of a workgroup per
     tile. Rows are scaled very differently, so a factor applied to the wrong row shows. K
-    beyond what a workgroup's waves hold stays with the other form."""
+    over 4,096 goes through a wave's registers in two halves; K beyond what a workgroup's
+    waves hold that way (5,120) stays with the other form."""
     hip, _ = kernel_sets[torch.bfloat16]
     y, w = rnd((M, K), torch.bfloat16, 50), rnd((d, K), torch.bfloat16, 51, K ** -0.5)
     res = rnd((M, d), torch.float32, 52) * torch.logspace(-2, 2, M, device=DEV)[:, None]

@@ -41,14 +41,14 @@ def test_key_splits_cases_that_used_to_exceed_the_limit():
 def test_a_sweep_shares_the_tiles_out_evenly():
     """At most one workgroup per compute unit (256), every workgroup the same number of weight
     tiles (tile pairs with SwiGLU) up to one, no workgroup without a tile; K beyond 16 waves
-    of 8 steps of 32 is refused. (The plan is host code of the product library; calling it
+    of two halves of 5 steps of 32 is refused. (The plan is host code of the product library; calling it
     needs the library, not a GPU.)"""
     from socrates_amd.kernels.build import load_library
     lib = load_library("gemm")
     lib.soc_gemm_sweep_plan.restype = c_int
     for swiglu in (0, 1):
         for N in (32, 64, 4096, 6144, 8192, 19456, 24576, 51200, 151936, 151968):
-            for K in (8, 64, 2560, 4096):
+            for K in (8, 64, 2560, 4096, 4104, 5120):
                 nw, wgs = c_int(0), c_int(0)
                 assert lib.soc_gemm_sweep_plan(c_int(N), c_int(K), c_int(swiglu), ctypes.byref(nw), ctypes.byref(wgs)) == 1
                 items = N // 32 if swiglu else (N + 15) // 16
@@ -57,7 +57,7 @@ def test_a_sweep_shares_the_tiles_out_evenly():
                 assert most == (items + 255) // 256                        # as few tiles for the busiest as 256 units allow
                 assert (most - 1) * wgs.value < items                      # nobody is idle
     nw, wgs = c_int(0), c_int(0)
-    for K in (4104, 5120, 9728):
+    for K in (5128, 8192, 9728):
         assert lib.soc_gemm_sweep_plan(c_int(2560), c_int(K), c_int(0), ctypes.byref(nw), ctypes.byref(wgs)) == 0
     # the shapes of a 4B-sized layer: 608 tile pairs as 203 x 3, 384 tiles as 192 x 2
     lib.soc_gemm_sweep_plan(c_int(19456), c_int(2560), c_int(1), ctypes.byref(nw), ctypes.byref(wgs))
