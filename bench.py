@@ -140,8 +140,9 @@ def decode_rate(engine, batch, context, steps, warmup, vocab, seed):
     import torch
     rng = random.Random(seed)
     from socrates_amd.sampling import SamplingParams
-    # requests whose prompt is done decode beside the portions of the others: room for that
-    portions = -(-context // engine.scheduler.token_budget)
+    # requests whose prompt is done decode beside the portions of the others, and take their
+    # share of a step's token budget: room for the tokens they generate meanwhile
+    portions = -(-context // max(1, engine.scheduler.token_budget - batch))
     params = SamplingParams(max_new_tokens=batch * portions + warmup + steps + 8, eos_token_ids=())
     reqs = [engine.submit([rng.randrange(vocab) for _ in range(context - 1)], sampling=params)
             for _ in range(batch)]
