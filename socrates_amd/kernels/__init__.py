@@ -86,7 +86,7 @@ def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, mi
     16 keys long, and cover keys 0 .. max_keys - 1. Host arithmetic only."""
     waves = n_blocks * n_kv_heads * ((group + 15) // 16)
     # from one wave per SIMD on (1,024) no split: a split costs a trip through LDS, or memory
-    n = 1 if waves >= max(1024, target_waves) else max(1, min((target_waves + waves - 1) // waves,
+    n = 1 if waves >= 1024 else max(1, min((target_waves + waves - 1) // waves,
                                            (max_keys + min_keys - 1) // min_keys, MAX_KEY_SPLITS))
     if n > 1:
         # splits that would each stream more than 2,048 keys are halved: twice the waves keep
