@@ -492,14 +492,15 @@ class HipKernels:
         """Workgroups that share one tile's K in ``linear_add_norm``: 1, 2 or 4, whichever gives
         the busiest of the GPU's 256 compute units the least to stream, with the meeting in
         memory priced at some 3,000 elements of K (less at more rows, where streaming is
-        slower); every wave keeps some 300 elements. Measured on an MI355X at the output and
+        slower); every wave keeps at least 256 elements. Measured on an MI355X at the output and
         down projections of 4B-, 8B- and 32B-sized layers (tiles 160, 256, 320; K 4,096 to
         25,600): 160 tiles of K = 9,728 take 12.3 us whole and 13.8 us in four parts at one row,
         15.6 and 15.3 us at 8 rows, 19.8 and 17.8 us at 16; 320 tiles of K = 25,600 take 77 us
-        whole and 56 us in four parts at 8 rows."""
+        whole and 56 us in four parts at 8 rows; 320 tiles of K = 8,192 take 24.4 us whole, 22.6 us
+        in two parts and 21.2 us in four at 8 rows."""
         best, best_cost = 1, None
         for splits in (1, 2, 4):
-            if splits > 1 and K // (splits * 8) < 300:
+            if splits > 1 and K // (splits * 8) < 256:
                 continue
             rounds = -(-tiles * splits // 256)
             cost = rounds * K / splits + (3000 * 8 / max(M, 8) if splits > 1 else 0)
