@@ -30,6 +30,9 @@ class ModelRunner:
         self._graph_max = 0
         self._graph_pool = None          # one memory pool for all captures: replays never overlap
         self.graphs_refused = None       # why enable_graphs left the steps eager, if it did
+        self._graph_epoch = 0            # the kernel set's ``graph_epoch`` the held graphs were captured under
+        if hasattr(model, "reserve"):
+            model.reserve(cache.max_len)     # tables by position stand at their final addresses from here on
         # eager steps: the batch's integers go through pinned staging memory, one copy per step
         self._upload = PinnedUploader(self.ops.device) if self.ops.device.type == "cuda" else None
 
@@ -99,6 +102,20 @@ class ModelRunner:
         self._graphs = {}
         self._graph_max = max_width
         self._graph_pool = torch.cuda.graph_pool_handle()
+        self._graph_epoch = getattr(self.ops, "graph_epoch", 0)
+
+    def _drop_stale_graphs(self) -> None:
+        """A captured step holds raw addresses and the choices of the kernel set at its
+        capture. The kernel set counts what takes either away (a table made anew, copies of
+        weights dropped, products tuned: ``graph_epoch``); graphs captured under another
+        count are dropped here and captured anew when a step needs them."""
+        epoch = getattr(self.ops, "graph_epoch", 0)
+        if epoch != self._graph_epoch:
+            if self._graphs:
+                torch.cuda.synchronize(self.ops.device)      # no replay is on its way when its graph goes
+                self._graphs.clear()
+                self._staging_read.clear()
+            self._graph_epoch = epoch
 
     def feeds(self, n_entries: int) -> bool:
         """Whether a step of ``n_entries`` single tokens can take them from the device
@@ -130,6 +147,7 @@ class ModelRunner:
         per graph."""
         if self._graphs is None:
             return 0
+        self._drop_stale_graphs()
         max_width = min(max_width or self._graph_max, self._graph_max)
         contexts, c = [], 256
         longest = min(max_context or self.cache.max_len, self.cache.max_len)
@@ -177,6 +195,7 @@ class ModelRunner:
             raise ValueError("a cache row appears twice in one step")
         if fed is not None and (fed.dtype != torch.int32 or fed.shape != (n,) or fed.device.type != self.ops.device.type):
             raise ValueError(f"fed tokens must be int32 [{n}] on {self.ops.device}")
+        self._drop_stale_graphs()
         width = self._bucket(n)
         # key splits of the attention kernel are planned per context bucket, so that a short
         # context is not cut into the many splits a long one needs

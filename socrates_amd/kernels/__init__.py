@@ -226,6 +226,14 @@ class HipKernels:
         # (the last to arrive leaves it so). All launches of this kernel set share them, so
         # they must not overlap: one stream, as everywhere in this package.
         self._split_count = torch.zeros(16384, dtype=torch.int32, device=self.device)
+        # Counts what takes away something a captured step relies on (an address it reads,
+        # a choice it was captured with); whoever holds graphs over this kernel set compares
+        # it with the count at their capture and drops them when it has moved.
+        self.graph_epoch = 0
+
+    def invalidate_graphs(self) -> None:
+        """Say that steps captured over this kernel set so far must not be replayed."""
+        self.graph_epoch += 1
 
     # -- helpers -----------------------------------------------------------------------------
     def _stream(self):
@@ -379,8 +387,11 @@ class HipKernels:
         return tiled, 1
 
     def forget_packed(self) -> None:
-        """Drop the copies by tile (to free memory). Graphs captured with this kernel set read
-        the copies by address: drop those first and capture anew afterwards."""
+        """Drop the copies by tile (to free memory). Steps captured with this kernel set read
+        the copies by address, so they are declared stale (``invalidate_graphs``): the runner
+        drops them before its next captured step and captures anew."""
+        if self._packed:
+            self.invalidate_graphs()
         self._packed.clear()
 
     def _sweep_plan(self, M, N, K, swiglu=False):
@@ -530,6 +541,7 @@ class HipKernels:
             tunable.set_numerical_check_tolerances(True, 1e-3, 8e-3)
         tunable.tuning_enable(bool(on))
         self._tuning = bool(on)
+        self.invalidate_graphs()                         # steps captured before replay the choices of their time
         if not on:
             self._cold = None                            # the buffer that cools the caches between timed calls
 

@@ -51,6 +51,12 @@ class PagedAttention:
         self.capturable = getattr(self.position, "capturable", True)
         self._free_layout = {"by_tile": True} if getattr(ops, "rows_by_tile", None) is not None else {}
 
+    def reserve(self, n_positions):
+        """Before the first step: what the position encoding keeps by position is made for
+        the cache's longest row."""
+        if hasattr(self.position, "reserve"):
+            self.position.reserve(n_positions)
+
     takes_projection = True     # the block may supply the last product
     takes_norm_owed = True      # x goes to one product only
 
@@ -65,7 +71,8 @@ class PagedAttention:
             Hkv = 0
         rot = self.position.rotary() if hasattr(self.position, "rotary") else None
         o = None
-        if (self.position is None or rot is not None) and hasattr(ops, "decode_attention"):
+        if ((self.position is None or rot is not None) and hasattr(ops, "decode_attention")
+                and ctx.max_q_len == 1):
             # a decode step: norm, position encoding, cache write and attention in one kernel
             table = self.position.table(ctx.max_ctx_len) if hasattr(self.position, "table") else None
             if self.position is None or table is not None:

@@ -67,6 +67,12 @@ class PreNormBlock:
         self.capturable = all(getattr(p, "capturable", True)
                               for p in (self.norm1, self.mixer, self.norm2, self.ffn))
 
+    def reserve(self, n_positions):
+        """Pass the cache's longest row on to the parts that keep something by position."""
+        for part in (self.norm1, self.mixer, self.norm2, self.ffn):
+            if hasattr(part, "reserve"):
+                part.reserve(n_positions)
+
     def _branch(self, part, args, residual, norm, consumer):
         """Run a mixer or feed-forward. If the part ends with a projection that it lets the
         block supply (``takes_projection``), the norm after it can be left to the kernel set

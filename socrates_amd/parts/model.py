@@ -56,6 +56,14 @@ class DecoderModel:
         self.capturable = (all(getattr(b, "capturable", True) for b in self.blocks)
                            and getattr(self.final_norm, "capturable", True))
 
+    def reserve(self, n_positions):
+        """Before the first step: parts that keep tables by position (a rotation's cosines
+        and sines) make them for ``n_positions``, the cache's longest row, so that they
+        stand at their final addresses when steps are captured."""
+        for block in self.blocks:
+            if hasattr(block, "reserve"):
+                block.reserve(n_positions)
+
     def forward(self, ctx, cache):
         """ctx: a StepContext on the device; cache: the CacheManager. Returns float32
         logits [len(ctx.want_index), vocab]."""

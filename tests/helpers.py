@@ -151,3 +151,55 @@ def replay(runner, steps):
             runner.cache.close_row(rows.pop(rid))
         runner.cache.check()
     return {rid: torch.cat(parts) for rid, parts in got.items()}
+
+
+def captured_decode_beside_a_long_prompt(runner, short, long_, want_short, want_long, close, first_decoded):
+    """A short request's decode step is captured for a small context bucket; then a prompt
+    that reaches far beyond it runs eagerly in portions, with other allocations between
+    the steps (whatever a captured step reads by address and a long step replaced would be
+    handed out again here); then the short request replays the step captured first.
+    ``want_*``: the plain implementation's logits for every position of the two requests;
+    ``close(got, want, what)`` compares. Every logit the engine computes is compared."""
+    import torch
+    from socrates_amd.engine import StepEntry
+    dev = runner.ops.device
+    a = runner.cache.open_row()
+    n = len(short)
+    mid = first_decoded + (n - first_decoded) // 2
+    got = runner.step([StepEntry(a, short[:first_decoded], [first_decoded - 1])]).float().cpu()
+    close(got[0], want_short[first_decoded - 1], "short request, end of its prompt")
+    for t in range(first_decoded, mid):
+        got = runner.step([StepEntry(a, short[t:t + 1], [0])]).float().cpu()
+        close(got[0], want_short[t], f"short request, decoded position {t} (first capture)")
+    bucket = runner._context_bucket(mid)
+    held = runner._graphs[(1, bucket)][0]
+    b = runner.cache.open_row()
+    junk = []
+    portion = (len(long_) + 2) // 3
+    for start in range(0, len(long_), portion):
+        tokens = long_[start:start + portion]
+        got = runner.step([StepEntry(b, tokens, [0, len(tokens) - 1])]).float().cpu()
+        close(got[0], want_long[start], f"long request, position {start}")
+        close(got[1], want_long[start + len(tokens) - 1], f"long request, position {start + len(tokens) - 1}")
+        # blocks of the sizes that tables and activations have, filled with what no cosine is
+        junk = [torch.full((s,), 3.0e4, dtype=torch.float32, device=dev) for s in (1 << 15, 1 << 17, 1 << 18, 1 << 19)]
+    del junk
+    for t in range(mid, n - 2):
+        got = runner.step([StepEntry(a, short[t:t + 1], [0])]).float().cpu()
+        close(got[0], want_short[t], f"short request, decoded position {t} (replayed after the long prompt)")
+    assert runner._graphs[(1, bucket)][0] is held, "the step captured first was not the one replayed"
+    # both requests in one captured step, whose positions reach as far as the long request's
+    c = runner.cache.open_row()
+    runner.step([StepEntry(c, long_[:len(long_) - 1], [])])
+    got = runner.step([StepEntry(a, short[n - 2:n - 1], [0]), StepEntry(c, long_[-1:], [0])]).float().cpu()
+    close(got[0], want_short[n - 2], "short request beside the long one")
+    close(got[1], want_long[len(long_) - 1], "long request, decoded last position")
+    assert (2, runner._context_bucket(len(long_))) in runner._graphs
+    junk = [torch.full((s,), 3.0e4, dtype=torch.float32, device=dev) for s in (1 << 15, 1 << 17, 1 << 18, 1 << 19)]
+    # and the short one alone again, from the step captured first (unless the kernel set
+    # said that it was stale: then from one captured anew)
+    got = runner.step([StepEntry(a, short[n - 1:], [0])]).float().cpu()
+    close(got[0], want_short[n - 1], "short request, last position, after a captured step that reached far")
+    del junk
+    for row in (a, b, c):
+        runner.cache.close_row(row)

@@ -114,7 +114,7 @@ def test_tuned_library_products_leave_the_tokens_alone(tmp_path, request):
     ops.fuse_norms = True
     for way in ("library", "own"):
         ops.product_choice = {k: way for k in ops.product_choice}
-        engine.runner._graphs = {}                       # captured steps hold the way they were captured with
+        ops.invalidate_graphs()                          # captured steps hold the way they were captured with
         got = engine.generate(prompts[:2])
         checked = [assert_same_where_clear(cfg, w, p, x, g) for p, g, x in zip(prompts, got, want)]
         assert checked[1] == 6, checked

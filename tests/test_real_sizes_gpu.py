@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from helpers import make_runner, random_prompts
+from helpers import captured_decode_beside_a_long_prompt, make_runner, random_prompts
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -100,3 +100,26 @@ def test_long_portion_beside_decoded_tokens(wide, dtype):
         close(logits[1:4], oracle[1][3 * j:3 * j + 3], dtype, f"step {j}: the long portion")
         close(logits[4], oracle[3][j], dtype, f"step {j}: decoded token of the 500-token request")
         close(logits[5], oracle[4][j], dtype, f"step {j}: decoded token of the 33-token request")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_captured_step_is_right_after_a_long_prompt(wide, dtype):
+    """Head size 128, a cache of 4,096 tokens: the 90-token request's decode step is captured
+    for contexts up to 256, the 2,200-token prompt then runs in three eager portions, and the
+    step captured first is replayed (the reference's captured steps read module buffers that
+    never move, model/qwen/qwen_kv_cont.py:97-127)."""
+    from socrates_amd.kernels import HipKernels
+    folder, cfg, w, prompts = wide
+    short, long_ = prompts[2], prompts[1]
+    want_short = plain.forward(cfg, w, short)
+    want_long = plain.forward(cfg, w, long_, rows=[0, 733, 734, 1467, 1468, 2199])
+    at = {0: 0, 733: 1, 734: 2, 1467: 3, 1468: 4, 2199: 5}
+
+    class Rows:                      # the oracle's rows of the long request, by position
+        def __getitem__(self, position):
+            return want_long[at[position]]
+
+    runner = make_runner(folder, HipKernels(dtype, DEV), max_rows=3, max_len=4096, block_size=16)
+    runner.enable_graphs(2)
+    captured_decode_beside_a_long_prompt(runner, short, long_, want_short, Rows(),
+                                         lambda got, want, what: close(got, want, dtype, what), first_decoded=70)
