@@ -10,6 +10,7 @@ is launched, so that a wrong operand is an exception and not a memory fault.
 
 from __future__ import annotations
 
+import collections
 import ctypes
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
@@ -230,6 +231,9 @@ class HipKernels:
         # a choice it was captured with); whoever holds graphs over this kernel set compares
         # it with the count at their capture and drops them when it has moved.
         self.graph_epoch = 0
+        # how often each form of a product or of the attention was launched (a replayed graph
+        # launches without coming by here): for tests and for whoever asks what a step ran
+        self.forms = collections.Counter()
 
     def invalidate_graphs(self) -> None:
         """Say that steps captured over this kernel set so far must not be replayed."""
@@ -348,6 +352,7 @@ class HipKernels:
                 n_waves //= 2
             ssq, tiles, dim, eps = self._owed_args(owed, M, K)
             wt, tiled = self._by_tile(w_gate_up)
+            self.forms["skinny_swiglu"] += 1
             _check(self._gemm.soc_gemm_bf16_skinny_swiglu(_ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N),
                                                           c_int(K), c_int(self.code), c_int(n_waves),
                                                           ssq, c_int(tiles), c_int(dim), c_float(eps),
@@ -413,6 +418,7 @@ class HipKernels:
         if ssq is not None:
             mode |= self._SK_SCALED
         wt, tiled = self._by_tile(w)
+        self.forms["sweep" + ("_swiglu" if mode & self._SK_SWIGLU else "")] += 1
         _check(self._gemm.soc_gemm_bf16_sweep(
             _ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(_DTYPE_CODE[out.dtype]), c_int(mode),
             c_int(plan[0]), c_int(plan[1]), ssq, c_int(tiles), c_int(dim), c_float(eps), c_int(tiled | layout),
@@ -435,6 +441,7 @@ class HipKernels:
         parts, kpw, groups = plan
         out = torch.empty((parts, M, N), dtype=torch.float32, device=self.device)
         wt, tiled = self._by_tile(w)
+        self.forms[f"parts_of_k:{parts}"] += 1
         _check(self._gemm.soc_gemm_bf16_sweep_parts(_ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K),
                                                     c_int(parts), c_int(kpw), c_int(groups), c_int(tiled),
                                                     self._stream()),
@@ -491,6 +498,7 @@ class HipKernels:
             sums = torch.empty((tiles, k_splits, 256), dtype=torch.float32, device=self.device)
             count = self._split_count
         wt, tiled = self._by_tile(w)
+        self.forms[f"add_norm:{k_splits}"] += 1
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(yx), _ptr(wt), None, c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(in_tiles),
             c_int(dim), c_float(in_eps), _ptr(residual), _ptr(gain), _ptr(x_out), _ptr(ssq_out),
@@ -604,6 +612,7 @@ class HipKernels:
                 choice = self.product_choice[key] = self._faster(
                     lambda: self.linear(x, w, out_dtype, allow_partial, -1), by_library)
             if choice == "library":
+                self.forms["library"] += 1
                 out = by_library()
                 return out.unsqueeze(0) if allow_partial else out
         explicit = row_tiles > 0 or n_waves or k_splits
@@ -640,12 +649,14 @@ class HipKernels:
                 out = torch.empty((M, N), dtype=out_dtype, device=self.device)
                 c_ptr, p_ptr = _ptr(out), None
             wt, tiled = self._by_tile(w) if M <= 16 else (w, 0)
+            self.forms[f"skinny:{k_splits}"] += 1
             _check(self._gemm.soc_gemm_bf16_skinny(_ptr(x), _ptr(wt), c_ptr, p_ptr, c_int(M), c_int(N), c_int(K),
                                                    c_int(_DTYPE_CODE[out_dtype]), c_int(row_tiles),
                                                    c_int(n_waves), c_int(k_splits), c_int(tiled), self._stream()),
                    f"linear [{M}x{K}] x [{N}x{K}]^T")
             return out
         if both_bf16 and self.library_gemm:
+            self.forms["library"] += 1
             if out_dtype == torch.bfloat16:
                 return torch.mm(x, w.t())
             return torch.mm(x, w.t(), out_dtype=out_dtype)
@@ -925,6 +936,7 @@ class HipKernels:
         tiled = bool(by_tile and self.rows_by_tile and N <= 16 and (Hq * D) % 32 == 0)
         out = torch.empty((Hq * D // 32, 16, 32) if tiled else (N, Hq * D), dtype=self.dtype, device=self.device)
         self.last_attention_kernel = ("fused", 1)
+        self.forms[f"fused_attention:{n_splits}"] += 1
         _check(lib.soc_paged_attention_decode_fused(
             _ptr(qkv), c_int(heads), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
             c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(out), _ptr(part_o),

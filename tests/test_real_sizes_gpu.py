@@ -123,3 +123,100 @@ def test_captured_step_is_right_after_a_long_prompt(wide, dtype):
     runner.enable_graphs(2)
     captured_decode_beside_a_long_prompt(runner, short, long_, want_short, Rows(),
                                          lambda got, want, what: close(got, want, dtype, what), first_decoded=70)
+
+
+# ---- the benchmark's own batch sizes -----------------------------------------------------------
+# Lengths on both sides of a page (16), of a 256-key context bucket and of the split plans; the
+# first 8, 16 and 24 of them each hold short and long ones.
+BATCH_LENGTHS = [19, 262, 35, 130, 255, 50, 257, 18, 100, 270, 31, 258, 66, 20, 200, 34,
+                 140, 259, 21, 36, 70, 256, 23, 260] + [24 + (7 * i) % 90 for i in range(40)]
+DECODED = 3       # tokens of every request that are decoded, all rows in one step
+
+
+def decode_rows_through_graphs(folder, cfg, w, prompts, want, dtype, live, expect_forms=()):
+    """``live`` requests: their prompts but the last DECODED tokens in eager steps, then those
+    tokens one per step, all rows in one captured step; every logit against ``want[i]``
+    [DECODED, V]. Returns the kernel set (its ``forms`` say what was launched)."""
+    from socrates_amd.engine import StepEntry
+    from socrates_amd.kernels import HipKernels
+    ops = HipKernels(dtype, DEV)
+    runner = make_runner(folder, ops, max_rows=live, max_len=512, block_size=16)
+    runner.enable_graphs(live)
+    rows = [runner.cache.open_row() for _ in range(live)]
+    for lo in range(0, live, 8):                                  # prompts, eight requests a step
+        runner.step([StepEntry(rows[i], prompts[i][:-DECODED], []) for i in range(lo, min(lo + 8, live))])
+    ops.forms.clear()
+    for t in range(DECODED):
+        batch = [StepEntry(rows[i], [prompts[i][len(prompts[i]) - DECODED + t]], [0]) for i in range(live)]
+        logits = runner.step(batch).float().cpu()
+        for i in range(live):
+            close(logits[i], want[i][t], dtype,
+                  f"{live} rows, step {t}, request {i} ({len(prompts[i])} tokens)")
+    assert all(k[0] == runner._bucket(live) for k in runner._graphs) and runner._graphs
+    for form in expect_forms:
+        assert any(k.startswith(form) for k in ops.forms), (form, dict(ops.forms))
+    return ops
+
+
+@pytest.fixture(scope="module")
+def wide_batch(wide):
+    folder, cfg, w, _ = wide
+    prompts = random_prompts(BATCH_LENGTHS, cfg["vocab_size"], seed=77)
+    want = [plain.forward(cfg, w, p, rows=list(range(len(p) - DECODED, len(p)))) for p in prompts]
+    return prompts, want
+
+
+@pytest.mark.parametrize("live", [8, 16, 24, 64])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_every_logit_at_the_benchmarks_batch_sizes(wide, wide_batch, dtype, live):
+    """The reference compares every logit of every step of its batched decode
+    (tests/test_paged_model.py:35-76). 8 and 16 rows: the sweep form of QKV, gate / up and the
+    head, the fused attention with key splits that meet in memory, rows handed on by tile, the
+    two projections with the residual sum and the next norm in their epilogue, chained over
+    both layers. 24 and 64 rows: library products beside the sweep over parts of K."""
+    folder, cfg, w, _ = wide
+    prompts, want = wide_batch
+    forms = () if dtype == torch.float32 else \
+        ("sweep", "sweep_swiglu", "add_norm", "fused_attention") if live <= 16 else ("parts_of_k", "library", "fused_attention")
+    ops = decode_rows_through_graphs(folder, cfg, w, prompts, want, dtype, live, forms)
+    if dtype == torch.bfloat16 and live == 8:
+        splits = [int(k.split(":")[1]) for k in ops.forms if k.startswith("fused_attention")]
+        assert max(splits) > 4, dict(ops.forms)              # the key splits met in memory
+
+
+# One or two layers at the widths of the larger models (random weights; a vocabulary of 8,192
+# keeps the head in the sweep form at K = 4,096 and 5,120).
+WIDER = {
+    "8b": dict(architectures=["Qwen3ForCausalLM"], vocab_size=8192, hidden_size=4096, num_hidden_layers=2,
+               num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288,
+               rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False),
+    "32b": dict(architectures=["Qwen3ForCausalLM"], vocab_size=8192, hidden_size=5120, num_hidden_layers=1,
+                num_attention_heads=64, num_key_value_heads=8, head_dim=128, intermediate_size=25600,
+                rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False),
+}
+
+
+@pytest.fixture(scope="module", params=["8b", "32b"])
+def wider(request, tmp_path_factory):
+    from socrates_amd.config import Qwen3Config
+    from socrates_amd.weights import write_random_model
+    folder = write_random_model(tmp_path_factory.mktemp(request.param) / "m", Qwen3Config.from_dict(WIDER[request.param]),
+                                31, dtype=torch.bfloat16, std=0.02, gain_std=0.1)
+    cfg, w = plain.read_folder(folder)
+    prompts = random_prompts(BATCH_LENGTHS[:40], cfg["vocab_size"], seed=78)
+    want = [plain.forward(cfg, w, p, rows=list(range(len(p) - DECODED, len(p)))) for p in prompts]
+    return request.param, folder, cfg, w, prompts, want
+
+
+@pytest.mark.parametrize("live", [1, 8, 40])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_layers_of_the_larger_models(wider, dtype, live):
+    """Widths 4,096 (K of 4,096 and 12,288) and 5,120 with 64 query heads (K of 5,120 in two
+    halves per wave, 8,192, and 25,600 split over four workgroups per tile): decode steps of
+    1, 8 and 40 rows through captured graphs, every logit against the plain implementation."""
+    name, folder, cfg, w, prompts, want = wider
+    forms = () if dtype == torch.float32 else \
+        ("sweep", "sweep_swiglu", "add_norm", "fused_attention") if live <= 16 else ("parts_of_k", "fused_attention")
+    ops = decode_rows_through_graphs(folder, cfg, w, prompts, want, dtype, live, forms)
+    if dtype == torch.bfloat16 and name == "32b" and live == 8:
+        assert ops.forms["add_norm:4"] >= 1, dict(ops.forms)     # K = 25,600 in four parts
