@@ -18,7 +18,7 @@ int soc_sample(const float* logits, const float* temperature, const long long* s
                const long long* draws, int* out, int n, int V, hipStream_t stream);
 
 // The same result as soc_argmax without a workspace argument and without any allocation.
-// It has no counterpart in the reference (which takes torch.argmax, model/inference_paged.py:166):
+// It has no counterpart in the reference:
 // it is for callers that cannot allocate device memory, such as code under HIP graph capture,
 // tight serving loops and harnesses that forbid hipMalloc. The chunk results live in a
 // file-scope device array of SOC_ARGMAX_STATIC_MAX_ROWS * SOC_ARGMAX_STATIC_MAX_CHUNKS pairs

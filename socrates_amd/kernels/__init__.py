@@ -780,6 +780,10 @@ class HipKernels:
     def plan_splits(self, n_tokens, n_kv_heads, group, max_keys):
         """How the keys of one token are cut into splits so that the launch fills the GPU."""
         if self.attention_splits is not None:
+            split_len, n_splits = self.attention_splits
+            if min(split_len, 1 << 24) * n_splits < max_keys:
+                raise KernelError(f"{n_splits} key splits of {split_len} keys do not cover the {max_keys} keys of the "
+                                  "step's longest row")
             return self.attention_splits
         chunk = 1 if group == 1 else 2 if group == 2 else 4 if group <= 4 else 8
         base = n_tokens * n_kv_heads * ((group + chunk - 1) // chunk)
@@ -836,6 +840,9 @@ class HipKernels:
         if self.attention_splits is not None:
             split_len, n_splits = self.attention_splits
             split_len = max(16, (min(split_len, 1 << 24) + 15) // 16 * 16)
+            if split_len * n_splits < max_keys:
+                raise KernelError(f"{n_splits} key splits of {split_len} keys do not cover the {max_keys} keys of the "
+                                  "step's longest row")
             n_splits = max(1, min(n_splits, (max_keys + split_len - 1) // split_len))
             if n_splits > 1:
                 n_splits = (n_splits + 3) // 4 * 4          # four splits share a workgroup

@@ -527,6 +527,126 @@ def test_decode_attention_from_raw_qkv(kernel_sets, Hq, Hkv, D, bs, norm, rope):
     assert hip.decode_attention(qkv[:, :(Hq + 2 * Hkv) * 32], Hq, Hkv, 32, None, None, 1e-6, table32, slot_a, ctx, 0.2) is None
 
 
+def plain_norm_rotate(x, gain, eps, positions, inv_freq):
+    """Per-head RMSNorm (x / sqrt(mean(x^2) + eps) * gain) and the rotate-half rotation of
+    x [N, H, D] in float32 on the CPU, rounded to bfloat16 once as a kernel's output is."""
+    x = x.float().cpu()
+    if gain is not None:
+        x = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain.cpu()
+    if inv_freq is not None:
+        ang = torch.tensor(positions, dtype=torch.float32)[:, None] * inv_freq.cpu()[None]
+        cos, sin = torch.cat([ang.cos()] * 2, -1)[:, None], torch.cat([ang.sin()] * 2, -1)[:, None]
+        h = x.shape[-1] // 2
+        x = x * cos + torch.cat([-x[..., h:], x[..., :h]], -1) * sin
+    return x.to(torch.bfloat16).float()
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,bs,rope", [(32, 8, 128, 16, True), (16, 1, 64, 32, True), (12, 3, 96, 8, False),
+                                              (6, 2, 128, 4, True)])
+@pytest.mark.parametrize("window", [None, 1, 16, 17, 40])
+def test_decode_attention_against_plain_attention(kernel_sets, Hq, Hkv, D, bs, rope, window):
+    """The one-kernel decode attention against plain float32 attention (norm, rotation and
+    softmax written out here, contiguous keys): lengths on both sides of a 16-key tile, of a
+    page and of the window; with and without key splits. For every row one early key is made
+    to win the softmax of one query head: the last key that the window hides (it must change
+    nothing) or, in a second pass, the first that it shows (the output is that key's value)."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    lens = [1, 15, 16, 17, 18, 33, 41, 48, 49, 300, 1025]
+    N, G, scale, eps = len(lens), Hq // Hkv, 0.2, 1e-6
+    rows, pos = list(range(N)), [n - 1 for n in lens]
+    g = torch.Generator().manual_seed(D + (window or 0))
+    q_gain = (1 + 0.3 * torch.randn(D, generator=g)).to(DEV)
+    k_gain = (1 + 0.3 * torch.randn(D, generator=g)).to(DEV)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, D, 2).float() / D))).to(DEV) if rope else None
+    table = hip.rope_table(inv_freq, 0, 1100) if rope else None
+    qkv = rnd((N, (Hq + 2 * Hkv) * D), torch.bfloat16, 61, 1.5)
+    heads = qkv.view(N, Hq + 2 * Hkv, D)
+    q = plain_norm_rotate(heads[:, :Hq], q_gain, eps, pos, inv_freq)
+    k_new = plain_norm_rotate(heads[:, Hq:Hq + Hkv], k_gain, eps, pos, inv_freq)
+    v_new = heads[:, Hq + Hkv:].float().cpu()
+    ctx = ctx_for(rows, pos)
+    for needle in ("hidden", "shown"):
+        slot, dense = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=D + 3)
+        planted = {}
+        for r, n in enumerate(lens):
+            k, v = dense[r]
+            k[:, n - 1], v[:, n - 1] = k_new[r], v_new[r]              # the token's own key and value
+            first = 0 if window is None else max(0, n - window)        # the first key the token sees
+            j = first - 1 if needle == "hidden" else first
+            if j < 0 or j >= n - 1:
+                continue                                               # (the token's own key comes from qkv)
+            h = (r % Hkv) * G                                          # a query head of kv head r % Hkv
+            key = (q[r, h] * (30.0 / (scale * float(q[r, h].pow(2).sum())))).to(torch.bfloat16)
+            k[r % Hkv, j] = key.float()
+            slot.k[int(slot.block_table[r, j // bs]), r % Hkv, j % bs] = key.to(DEV)
+            planted[r] = (h, j)
+        want = dense_attention(q.to(torch.bfloat16), dense, rows, pos, scale, window)
+        if needle == "shown":
+            for r, (h, j) in planted.items():                          # the oracle itself saw the needle
+                assert (want[r].view(Hq, D)[h] - dense[r][1][r % Hkv, j]).abs().max() < 0.02
+        for splits in (None, (16, 68), (64, 17), (1 << 30, 1)):
+            hip.attention_splits = splits
+            pages = (slot.k.clone(), slot.v.clone())
+            got = hip.decode_attention(qkv, Hq, Hkv, D, q_gain, k_gain, eps, table, slot, ctx, scale, window, True)
+            assert got is not None
+            close(got.cpu(), want, torch.bfloat16)
+            slot.k.copy_(pages[0]), slot.v.copy_(pages[1])
+        hip.attention_splits = None
+        if window not in (None, 1):
+            assert len(planted) >= 5            # rows long enough to have a key on that side of the window's edge
+    hip.attention_splits = (16, 8)              # splits that do not reach the longest row's last key are refused
+    with pytest.raises(Exception, match="do not cover"):
+        hip.decode_attention(qkv, Hq, Hkv, D, q_gain, k_gain, eps, table, slot, ctx, scale, window, True)
+    hip.attention_splits = None
+    assert int(hip._split_count.abs().sum()) == 0
+
+
+def test_workgroups_that_meet_in_memory_give_the_same_bits_every_time(kernel_sets):
+    """The decode attention with more than four key splits and the projection with the
+    residual epilogue whose K is shared by four workgroups exchange partial results through
+    memory inside one launch, ordered by an arrival count and no fence. A partial result read
+    before it had arrived would change the sum: the same launch, repeated a few hundred times
+    on one input, has to give the same bits every time and leave the counts at zero. Stops at
+    the first difference."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    # attention: 8 rows of 8 kv heads, 2,048 keys each, 16 splits (the benchmark's decode step)
+    Hq, Hkv, D, bs, N = 32, 8, 128, 16, 8
+    lens = [2048 - 37 * r for r in range(N)]
+    slot, _ = make_paged_case(lens, Hq, Hkv, D, bs, torch.bfloat16, seed=4)
+    rows, pos = list(range(N)), [n - 1 for n in lens]
+    ctx = ctx_for(rows, pos)
+    qkv = rnd((N, (Hq + 2 * Hkv) * D), torch.bfloat16, 62)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, D, 2).float() / D))).to(DEV)
+    table = hip.rope_table(inv_freq, 0, 2048)
+    gain = torch.ones(D, device=DEV)
+    hip.forms.clear()
+    first = None
+    for i in range(300):
+        got = hip.decode_attention(qkv, Hq, Hkv, D, gain, gain, 1e-6, table, slot, ctx, D ** -0.5, None, True)
+        if first is None:
+            first = got.clone()
+            assert max(int(k.split(":")[1]) for k in hip.forms if k.startswith("fused_attention")) > 4
+        elif not torch.equal(got, first):
+            raise AssertionError(f"decode attention, launch {i}: {int((got != first).sum())} values differ from the first launch")
+    assert int(hip._split_count.abs().sum()) == 0
+    # the down projection of a 32B-sized layer at 8 rows: four workgroups per tile of 16 outputs
+    M, Nout, K = 8, 5120, 25600
+    y, w = rnd((M, K), torch.bfloat16, 63, 0.5), rnd((Nout, K), torch.bfloat16, 64, 0.02)
+    norm_gain = (1 + 0.1 * torch.randn(Nout)).to(DEV)
+    residual = rnd((M, Nout), torch.float32, 65)
+    hip.forms.clear()
+    first = None
+    for i in range(200):
+        res = residual.clone()
+        owed = hip.linear_add_norm(y, w, res, norm_gain, 1e-6)
+        if first is None:
+            first = (owed.x.clone(), owed.ssq.clone(), res.clone())
+            assert hip.forms["add_norm:4"] == 1, dict(hip.forms)
+        elif not (torch.equal(owed.x, first[0]) and torch.equal(owed.ssq, first[1]) and torch.equal(res, first[2])):
+            raise AssertionError(f"linear_add_norm, launch {i}: the result differs from the first launch")
+    assert int(hip._split_count.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     """Tokens of one row at consecutive positions (a portion that starts mid-sequence)

@@ -72,10 +72,55 @@ def test_attention_reduces_to_the_library_routine():
     # q = 0: uniform weights, the output is the running mean of V
     mean = torch.cumsum(v, 0) / torch.arange(1, T + 1)[:, None, None]
     torch.testing.assert_close(plain.attention_scores(torch.zeros_like(q), k, v, 0.3), mean, atol=1e-5, rtol=1e-5)
-    # softmax is shift invariant: adding a constant to all scores of a query changes nothing
-    k2 = k.clone()
-    torch.testing.assert_close(plain.attention_scores(q, k2, v, 0.3),
-                               plain.attention_scores(q, k2, v + 0.0, 0.3))
+    # softmax is shift invariant: one more coordinate, 1 in every query and c in every key, adds
+    # 0.3 c to all scores of a query and changes nothing (an unnormalised or overflowing exp would)
+    for c in (5.0, -200.0, 200.0):
+        q1 = torch.cat([q, torch.ones(T, H, 1)], -1)
+        k1 = torch.cat([k, torch.full((T, H, 1), c)], -1)
+        v1 = torch.cat([v, torch.zeros(T, H, 1)], -1)
+        shifted = plain.attention_scores(q1, k1, v1, 0.3)
+        torch.testing.assert_close(shifted[..., :D], want, atol=1e-5, rtol=1e-5)
+    # and a shift that differs from key to key is not: the check above can fail
+    k1[3:, :, -1] += 4.0
+    assert not torch.allclose(plain.attention_scores(q1, k1, v1, 0.3)[..., :D], want, atol=1e-3)
+
+
+def test_attention_layer_takes_the_library_routines_default_scale(tmp_path):
+    """The reference's prompt pass hands q, k, v to the library's attention without a scale
+    (model/qwen/qwen_kv_paged.py:171-173), whose default is 1 / sqrt(last dimension of q); its
+    decode pass passes head_dim ** -0.5 to its own kernel (:139). The plain layer against the
+    same layer put together from library routines, with no scale written anywhere, at a head
+    size (32) that is neither hidden / heads (12) nor one at which 1 / sqrt(D) and 1 / D or 1
+    give like results: the scores are several units wide."""
+    folder = write_tiny(tmp_path / "B", TINY_B, seed=4)
+    cfg, w = plain.read_folder(folder)
+    T, Hq, Hkv, D = 19, cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    assert D == 32 and cfg["hidden_size"] // Hq == 12
+    p = "model.layers.1.self_attn."
+    x = 3.0 * torch.randn(T, cfg["hidden_size"])
+    pos = torch.arange(T)
+    q = F.rms_norm((x @ w[p + "q_proj.weight"].T).view(T, Hq, D), (D,), 4.0 * w[p + "q_norm.weight"], cfg["rms_norm_eps"])
+    k = F.rms_norm((x @ w[p + "k_proj.weight"].T).view(T, Hkv, D), (D,), w[p + "k_norm.weight"], cfg["rms_norm_eps"])
+    v = (x @ w[p + "v_proj.weight"].T).view(T, Hkv, D)
+    # the rotation as a complex multiplication of (x[j], x[j + D/2]) by exp(i position inv_freq[j])
+    inv_freq = 1.0 / (cfg["rope_theta"] ** (torch.arange(0, D, 2).float() / D))
+    turn = torch.polar(torch.ones(T, D // 2), pos[:, None].float() * inv_freq)[:, None]
+    def rotate(t):
+        z = torch.complex(t[..., :D // 2], t[..., D // 2:]) * turn
+        return torch.cat([z.real, z.imag], -1)
+    o = F.scaled_dot_product_attention(rotate(q).transpose(0, 1)[None], rotate(k).transpose(0, 1)[None],
+                                       v.transpose(0, 1)[None], is_causal=True, enable_gqa=True)[0]
+    want = o.transpose(0, 1).reshape(T, Hq * D) @ w[p + "o_proj.weight"].T
+    w4 = dict(w)
+    w4[p + "q_norm.weight"] = 4.0 * w[p + "q_norm.weight"]           # sharper scores: the scale shows
+    got = plain.attention_layer(x, w4, p, cfg, pos)
+    torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-4)
+    # the same routine with the scales a misreading would give is far away
+    for wrong in (1.0 / D, 1.0, (cfg["hidden_size"] // Hq) ** -0.5):
+        o = F.scaled_dot_product_attention(rotate(q).transpose(0, 1)[None], rotate(k).transpose(0, 1)[None],
+                                           v.transpose(0, 1)[None], is_causal=True, enable_gqa=True, scale=wrong)[0]
+        other = o.transpose(0, 1).reshape(T, Hq * D) @ w[p + "o_proj.weight"].T
+        assert (other - want).abs().max() > 50 * (got - want).abs().max() + 1e-3
 
 
 def test_attention_needles_fix_length_bound_and_head_mapping():

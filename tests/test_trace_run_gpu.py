@@ -45,8 +45,10 @@ def build_trace(prompts):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("tiny,seed", [(TINY_A, 1), (TINY_B, 2)], ids=["A", "B"])
-def test_trace_run_matches_plain(tmp_path, tiny, seed, dtype):
+@pytest.mark.parametrize("tiny,seed,options", [(TINY_A, 1, []), (TINY_B, 2, []),
+                                               (TINY_B, 2, ["--block-size", "8", "--max-rows", "4"])],
+                         ids=["A", "B", "B-pages-of-8"])
+def test_trace_run_matches_plain(tmp_path, tiny, seed, options, dtype):
     folder = write_tiny(tmp_path / "model", tiny, seed=seed)
     cfg, w = plain.read_folder(folder)
     prompts = random_prompts([5, 33, 70, 64, 100, 41], cfg["vocab_size"], seed=seed)
@@ -56,7 +58,7 @@ def test_trace_run_matches_plain(tmp_path, tiny, seed, dtype):
     max_tokens = sum(-(-len(p) // 64) * 64 for p in sorted(prompts, key=len)[-4:])
     out = tmp_path / "out"
     proc = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype,
-                           "--out", str(out), "--max-tokens", str(max_tokens)],
+                           "--out", str(out), "--max-tokens", str(max_tokens)] + options,
                           input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert proc.stdout.split("\n")[:-1] == [f"done {i}" for i in range(len(lines))]
