@@ -183,6 +183,58 @@ def prefill_rate(engine, tokens, vocab, seed, repeats=3):
     return best
 
 
+def release(engine):
+    """Give an engine's memory back (weights, cache, captured steps) before the next is built."""
+    import gc
+
+    import torch
+    engine.runner._graphs = None
+    engine.runner.model = engine.runner.cache = None
+    engine.cache = engine.sampler = engine.scheduler = None
+    del engine
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def other_sizes(args, dtype, item):
+    """Decode at batch 8 at longer contexts, and decode and a 2,048-token prefill at the larger
+    models' layer sizes: flat entries for ``points``, each rate with the fraction of its
+    roofline (decode: bytes read over 8 TB/s; prefill: flops over the dtype's peak)."""
+    import torch
+    out = {}
+
+    def decode_point(name, config, engine, batch, context):
+        tok_s, ms = decode_rate(engine, batch, context, 16, 4, config.vocab_size, seed=11)
+        step_bytes = (config.param_counts()["read_per_step"] * item
+                      + batch * context * config.kv_bytes_per_token(item))
+        out[name] = round(tok_s, 1)
+        out[name + "_ms"] = round(ms, 4)
+        out[name + "_hbm_frac"] = round(step_bytes / (ms * 1e-3) / 1e9 / HBM_GBPS, 4)
+
+    # the headline model behind longer contexts
+    cfg = preset_dict(DEFAULT_PRESET)
+    config, engine = build_engine(cfg, dtype, 8, 32768 + 512, seed=0, compile_=not args.no_graphs,
+                                  block_size=args.block_size)
+    for context in (8192, 32768):
+        decode_point(f"decode_b8_ctx{context}", config, engine, 8, context)
+    release(engine)
+    # the larger models: all layers of each, the contexts that BASELINE.json gives them
+    for tag, preset, context in (("8b", "qwen3-8b", 2048), ("32b", "qwen3-32b", 8192)):
+        cfg = preset_dict(preset)
+        config, engine = build_engine(cfg, dtype, 8, context + 512, seed=0, compile_=not args.no_graphs,
+                                      block_size=args.block_size)
+        if args.dtype == "bf16" and not args.no_tune:
+            engine.tune([args.prefill_tokens])
+        decode_point(f"decode_b8_{tag}_ctx{context}", config, engine, 8, context)
+        pre_s = prefill_rate(engine, args.prefill_tokens, config.vocab_size, seed=12, repeats=2)
+        out[f"prefill_{tag}_ms"] = round(pre_s * 1e3, 3)
+        out[f"prefill_{tag}_frac"] = round(config.prefill_flops(args.prefill_tokens) / pre_s / PEAK_FLOPS[args.dtype], 4)
+        out[f"layers_{tag}"] = config.num_hidden_layers
+        release(engine)
+        torch.cuda.synchronize()
+    return out
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +255,8 @@ def main(argv=None):
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-sizes", action="store_true",
+                    help="skip the points at longer contexts and at the larger models' layer sizes")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-tune", action="store_true", help="library products with the library's default choice")
     ap.add_argument("--split-waves", type=int, default=None, help="key splits of the decode attention: waves aimed at")
@@ -264,6 +318,9 @@ def main(argv=None):
         for b in (1, 64):
             points[f"decode_b{b}"] = round(decode_rate(engine, b, args.context, max(8, args.steps // 2),
                                                        4, V, seed=3 + b)[0], 1)
+    if not args.no_points and not args.no_sizes and args.preset == DEFAULT_PRESET and args.layers == full_layers:
+        release(engine)
+        points.update(other_sizes(args, dtype, item))
     out = {
         "metric": f"decode tok/s @ batch {args.batch}, context {args.context} ({sized}, {args.dtype})",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
