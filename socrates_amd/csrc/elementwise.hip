@@ -115,7 +115,7 @@ __global__ void __launch_bounds__(1024)
 add_rmsnorm_vec8_kernel(float* __restrict__ residual, const T* __restrict__ delta,
                         const float* __restrict__ partials, int n_partials, size_t partial_stride,
                         const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
-                        int d, float eps) {
+                        int d, float eps, int tile_rows) {
     __shared__ float scratch[16];
     const int i = blockIdx.x;
     const int n = rows ? rows[i] : i;
@@ -154,7 +154,9 @@ add_rmsnorm_vec8_kernel(float* __restrict__ residual, const T* __restrict__ delt
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);
     if (!in) return;
-    T* o = out + (size_t)i * d + j;
+    // tile_rows R > 0 (d a multiple of 32): out is laid out [d / 32][R][32] for a product that
+    // reads 64 bytes of each of its rows side by side
+    T* o = tile_rows > 0 ? out + ((size_t)(j / 32) * tile_rows + i) * 32 + j % 32 : out + (size_t)i * d + j;
     if constexpr (sizeof(T) == 2) {
         uint4 pk;
         pk.x = pack_bf16x2(v[0] * inv * g[0], v[1] * inv * g[1]);
@@ -170,36 +172,40 @@ add_rmsnorm_vec8_kernel(float* __restrict__ residual, const T* __restrict__ delt
 }
 
 template <typename T>
-static void launch_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
-                               size_t partial_stride, const float* w, void* out, const int* rows, int n_out,
-                               int d, float eps, hipStream_t stream) {
+static int launch_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
+                              size_t partial_stride, const float* w, void* out, const int* rows, int n_out,
+                              int d, float eps, int tile_rows, hipStream_t stream) {
     constexpr int VPT = 8;
     const int threads = d <= 1024 ? 128 : (d <= 2048 ? 256 : (d <= 4096 ? 512 : 1024));
     const bool aligned = d % 8 == 0 && partial_stride % 4 == 0 &&
                          ((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)partials | (uintptr_t)w | (uintptr_t)out) % 16 == 0;
+    if (tile_rows > 0 && !(aligned && d <= 8 * 1024 && d % 32 == 0 && n_out <= tile_rows))
+        return (int)hipErrorInvalidValue;                // only the 16-byte form lays its output out by tile
     if (aligned && d <= 8 * 1024)
         hipLaunchKernelGGL(add_rmsnorm_vec8_kernel<T>, dim3(n_out), dim3((d / 8 + 63) / 64 * 64), 0, stream, residual,
-                           (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
+                           (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps, tile_rows);
     else if (d <= VPT * threads)
         hipLaunchKernelGGL((add_rmsnorm_regs_kernel<T, VPT>), dim3(n_out), dim3(threads), 0, stream, residual,
                            (const T*)delta, partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(1024), 0, stream, residual, (const T*)delta,
                            partials, n_partials, partial_stride, w, (T*)out, rows, d, eps);
+    return 0;
 }
 
+// tile_rows R > 0: out is written [d / 32][R][32] (R >= n_out; d a multiple of 32, at most 8,192,
+// 16-byte aligned operands) instead of [n_out][d].
 SOC_EXPORT int soc_add_rmsnorm(float* residual, const void* delta, const float* partials, int n_partials,
                                long long partial_stride, const float* w, void* out, const int* rows,
-                               int n_out, int d, float eps, int dtype, hipStream_t stream) {
+                               int n_out, int d, float eps, int dtype, int tile_rows, hipStream_t stream) {
     if (n_out <= 0) return 0;
     if (delta && partials) return (int)hipErrorInvalidValue;
-    if (dtype == 0)
-        launch_add_rmsnorm<float>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
-                                  n_out, d, eps, stream);
-    else
-        launch_add_rmsnorm<bf16>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
-                                 n_out, d, eps, stream);
-    return soc_last_error();
+    const int refused = dtype == 0
+        ? launch_add_rmsnorm<float>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
+                                    n_out, d, eps, tile_rows, stream)
+        : launch_add_rmsnorm<bf16>(residual, delta, partials, n_partials, (size_t)partial_stride, w, out, rows,
+                                   n_out, d, eps, tile_rows, stream);
+    return refused ? refused : soc_last_error();
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -1078,3 +1078,189 @@ SOC_EXPORT int soc_gemm_bf16_sweep_parts(const void* X, const void* W, float* P,
 #undef SOC_SWP
     return soc_last_error();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Products of 17 to 64 rows whose consumer wants whole sums (QKV, gate / up with its activation,
+// the output head): K outermost. The sweeps above keep a wave's slices of x in registers and
+// walk over weight tiles, which ends at 16 rows of K = 5,120; with more rows x does not fit, and
+// a workgroup that re-reads it per tile brings more of x than of the weights into its compute
+// unit. Here a workgroup (at most one per compute unit, 8 waves) owns up to T weight tiles
+// per pass and keeps their sums, not x, in registers: round r of the walk over K gives wave w
+// the 32 k of step 8 r + w, for which it loads MT slices of x (its rows, used for all T tiles
+// and never again) and T slices of weights, and multiplies. x thus enters a compute unit once
+// per pass and goes through no LDS; the weights of two rounds are on their way at any time.
+// At the end of K the eight waves' sums of a tile meet in LDS (one barrier per tile) and the
+// workgroup's threads add them and write the outputs, with the activation for a pair of
+// gate and up tiles. A workgroup with more than T tiles takes further passes (x is read
+// again in each).
+struct StPlan {
+    int items;                      // weight tiles (tile pairs with SWIGLU)
+    int per_wg;                     // items of a workgroup: g, g + G, ...
+};
+
+template <typename TC, int MT, int T, int MODE>
+__global__ void __launch_bounds__(512)
+gemm_bf16_stream_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C, int M,
+                        int N, int K, StPlan pl, int layout) {
+    constexpr bool SWIGLU = MODE & SK_SWIGLU;
+    constexpr int SUB = SWIGLU ? 2 : 1, J = T / SUB, NW = 8;
+    static_assert(T % SUB == 0, "whole pairs");
+    const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED;
+    __shared__ __attribute__((aligned(16))) float red[2][NW][MT][256];   // [tile parity][wave][row block][lane][4]
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
+    const int g = blockIdx.x, G = gridDim.x;
+    const int li = lane % 16, lk = (lane / 16) * 8;
+    const int steps = (K + 31) / 32, rounds = (steps + NW - 1) / NW;
+    // x row by row [M][K], or by tile [K / 32][16 MT][32] (rows from M on hold anything: their
+    // sums are never stored)
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, (x_tiled ? 16 * MT : M) * K * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(W), (short)0, (int)((size_t)N * K * 2), 0x00020000);
+    const int w_rs = w_tiled ? 32 : K, w_ss = w_tiled ? 512 : 32;
+    const int x_rs = x_tiled ? 32 : K, x_ss = x_tiled ? 16 * MT * 32 : 32;
+
+    for (int pass = 0; pass * J < pl.per_wg; ++pass) {
+        // this pass's tiles: byte offset of each tile's first row, or nowhere
+        uint32_t tile_at[T];
+        int tile_no[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int j = pass * J + t / SUB, item = g + j * G;
+            const bool live = j < pl.per_wg && item < pl.items;
+            tile_no[t] = live ? (SWIGLU ? 2 * item + t % SUB : item) : -1;
+            tile_at[t] = live ? (uint32_t)((size_t)tile_no[t] * 16 * K * 2) : SW_NOWHERE;
+        }
+        if (tile_no[0] < 0) break;                          // the same in the whole workgroup
+        f32x4 acc[T][MT];
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int b = 0; b < MT; ++b) acc[t][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        // Loads of round r: nothing touches what they bring before their products (no branch
+        // around a load, no select on its result); a slice beyond K, a tile beyond the
+        // workgroup's share and a row beyond M are asked of nowhere and read as zeros.
+        auto load = [&](int r, uint4 (&wb)[T], uint4 (&xb)[MT]) {
+            const int step = r * NW + wave, k = step * 32 + lk;
+            const bool ok = r < rounds && k < K;
+            const uint32_t k_off = (uint32_t)(((step * w_ss) + li * w_rs + lk) * 2);
+#pragma unroll
+            for (int b = 0; b < MT; ++b)
+                xb[b] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                            x_rsrc, ok ? (uint32_t)((step * x_ss + (b * 16 + li) * x_rs + lk) * 2) : SW_NOWHERE, 0, 0));
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+                wb[t] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                            w_rsrc, ok && tile_at[t] != SW_NOWHERE ? tile_at[t] + k_off : SW_NOWHERE, 0, 0));
+        };
+        auto multiply = [&](const uint4 (&wb)[T], const uint4 (&xb)[MT]) {
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int b = 0; b < MT; ++b)
+                    acc[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wb[t]),
+                                                                        __builtin_bit_cast(bf16x8, xb[b]), acc[t][b], 0, 0, 0);
+        };
+        uint4 wa[T], xa[MT], wb2[T], xb2[MT];
+        load(0, wa, xa);
+        load(1, wb2, xb2);
+        for (int r = 0; r < rounds; r += 2) {
+            multiply(wa, xa);
+            load(r + 2, wa, xa);
+            multiply(wb2, xb2);
+            load(r + 3, wb2, xb2);
+        }
+        // The waves' sums of one tile at a time through LDS. acc[e] of lane l is row l % 16 of
+        // the block and column 4 (l / 16) + e of the tile. A thread adds the eight waves' sums
+        // of two neighbouring columns of one row: thread i takes row i / 8 of the MT * 16 and
+        // columns 2 (i % 8), + 1.
+        float held[2] = {0.f, 0.f};                          // SWIGLU: the gate sums, until the up sums are there
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int p = t % 2;
+#pragma unroll
+            for (int b = 0; b < MT; ++b)
+                *reinterpret_cast<float4*>(&red[p][wave][b][lane * 4]) =
+                    make_float4(acc[t][b][0], acc[t][b][1], acc[t][b][2], acc[t][b][3]);
+            __syncthreads();
+            if (tile_no[t] < 0) continue;                    // the same in the whole workgroup
+            for (int i = tid; i < MT * 16 * 8; i += 512) {
+                const int m = i / 8, c2 = (i % 8) * 2;
+                const int at = ((c2 / 4) * 16 + m % 16) * 4 + c2 % 4;
+                float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float2 v = *reinterpret_cast<const float2*>(&red[p][w][m / 16][at]);
+                    s0 += v.x; s1 += v.y;
+                }
+                if constexpr (SWIGLU) {
+                    if (t % 2 == 0) { held[0] = s0; held[1] = s1; continue; }
+                    const int col = (tile_no[t] / 2) * 16 + c2, half = N / 2;
+                    if (m < M && col < half) {
+                        const float a0 = s0 * (held[0] / (1.0f + expf(-held[0])));
+                        const float a1 = s1 * (held[1] / (1.0f + expf(-held[1])));
+                        C[(size_t)m * half + col] = from_float<TC>(a0);
+                        if (col + 1 < half) C[(size_t)m * half + col + 1] = from_float<TC>(a1);
+                    }
+                } else {
+                    const int n = tile_no[t] * 16 + c2;
+                    if (m < M && n < N) {
+                        C[(size_t)m * N + n] = from_float<TC>(s0);
+                        if (n + 1 < N) C[(size_t)m * N + n + 1] = from_float<TC>(s1);
+                    }
+                }
+            }
+        }
+        __syncthreads();                                     // the next pass writes `red` again
+    }
+}
+
+// Shape of such a product: workgroups and items (tiles, or tile pairs with SWIGLU) per
+// workgroup; 0 if the form does not apply.
+SOC_EXPORT int soc_gemm_stream_plan(int M, int N, int K, int swiglu, int* workgroups, int* per_wg) {
+    if (M < 1 || M > 64 || N < 1 || K < 8 || K % 8) return 0;
+    if (swiglu && N % 32) return 0;
+    const int items = swiglu ? N / 32 : (N + 15) / 16;
+    const int per = (items + 255) / 256;
+    *per_wg = per;
+    *workgroups = (items + per - 1) / per;
+    return 1;
+}
+
+// C = X [M <= 64, K] times W [N, K] transposed, in c_dtype (0 float32, 1 bfloat16), or with
+// mode SK_SWIGLU C [M, N / 2] = silu(gate) * up over weight rows that alternate in blocks of 16
+// (bfloat16 out). layout: SK_W_TILED, and SK_X_TILED: x is laid out [K / 32][R][32] with R = 32 for
+// M <= 32, 48 for M <= 48 and 64 above (K a multiple of 32). The matrices lie below 4 GiB.
+SOC_EXPORT int soc_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
+                                    int mode, int workgroups, int per_wg, int layout, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if ((layout & ~(SK_W_TILED | SK_X_TILED)) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) ||
+        ((layout & SK_X_TILED) && K % 32))
+        return (int)hipErrorInvalidValue;
+    if (M > 64 || K % 8 || K < 8 || !C) return (int)hipErrorInvalidValue;
+    if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull || (size_t)64 * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;
+    const bool swiglu = mode & SK_SWIGLU;
+    if ((mode & ~SK_SWIGLU) || (swiglu && (N % 32 || c_dtype != 1))) return (int)hipErrorInvalidValue;
+    if (c_dtype != 0 && c_dtype != 1) return (int)hipErrorInvalidValue;
+    StPlan pl;
+    pl.items = swiglu ? N / 32 : (N + 15) / 16;
+    if (workgroups < 1 || per_wg < 1 || (long)workgroups * per_wg < pl.items) return (int)hipErrorInvalidValue;
+    pl.per_wg = per_wg;
+    const dim3 grid(workgroups < pl.items ? workgroups : pl.items), block(512);
+    const int tiles_wg = per_wg * (swiglu ? 2 : 1);          // tiles of a workgroup: as many per pass as fit
+    const int T = tiles_wg <= 2 ? 2 : tiles_wg <= 4 ? 4 : tiles_wg % 6 == 0 || tiles_wg > 8 ? 6 : 4;
+#define SOC_ST(TC_, MT_, T_, MODE_) \
+    hipLaunchKernelGGL((gemm_bf16_stream_kernel<TC_, MT_, T_, MODE_>), grid, block, 0, stream, (const bf16*)X, \
+                       (const bf16*)W, (TC_*)C, M, N, K, pl, layout)
+#define SOC_ST_T(TC_, MT_, MODE_) \
+    do { if (T == 2) SOC_ST(TC_, MT_, 2, MODE_); else if (T == 4) SOC_ST(TC_, MT_, 4, MODE_); else SOC_ST(TC_, MT_, 6, MODE_); } while (0)
+#define SOC_ST_MT(TC_, MODE_) \
+    do { if (M <= 32) SOC_ST_T(TC_, 2, MODE_); else if (M <= 48) SOC_ST_T(TC_, 3, MODE_); else SOC_ST_T(TC_, 4, MODE_); } while (0)
+    if (swiglu) SOC_ST_MT(bf16, SK_SWIGLU);
+    else if (c_dtype == 1) SOC_ST_MT(bf16, 0);
+    else SOC_ST_MT(float, 0);
+#undef SOC_ST_MT
+#undef SOC_ST_T
+#undef SOC_ST
+    return soc_last_error();
+}

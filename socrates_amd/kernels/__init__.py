@@ -40,7 +40,7 @@ def _check(err, what):
 P, I, F = c_void_p, c_int, c_float
 _EW_SIGNATURES = {
     "soc_embedding": [P, P, P, I, I, I, I, P],
-    "soc_add_rmsnorm": [P, P, P, I, c_longlong, P, P, P, I, I, F, I, P],
+    "soc_add_rmsnorm": [P, P, P, I, c_longlong, P, P, P, I, I, F, I, I, P],
     "soc_rmsnorm": [P, P, P, I, I, F, I, P],
     "soc_swiglu": [P, P, I, I, I, I, P],
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
@@ -59,6 +59,8 @@ _GEMM_SIGNATURES = {
     "soc_gemm_sweep_plan": [I, I, I, P, P],
     "soc_gemm_bf16_sweep_parts": [P, P, P, I, I, I, I, I, I, I, P],
     "soc_gemm_sweep_parts_plan": [I, I, I, P, P, P],
+    "soc_gemm_bf16_stream": [P, P, P, I, I, I, I, I, I, I, I, P],
+    "soc_gemm_stream_plan": [I, I, I, I, P, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
@@ -121,13 +123,14 @@ class NormOwed:
 
 
 class RowsByTile:
-    """At most 16 rows of bfloat16 activations laid out by tile, ``data`` [dim / 32, 16, 32]
-    (element (row, col) at [col // 32, row, col % 32]; rows from ``rows`` on are never written
-    or read), for the product that takes them next: it then asks the L2 for one piece of
-    rows x 64 bytes per load where rows laid out one after the other give it that many pieces.
-    Made by ``decode_attention`` and ``linear_swiglu`` where the caller allows it (``by_tile``:
-    the caller hands the result to ``linear_add_norm`` or ``linear`` and nowhere else), taken
-    by those two."""
+    """Rows of bfloat16 activations laid out by tile, ``data`` [dim / 32, R, 32] with R the rows
+    rounded up to a multiple of 16 (element (row, col) at [col // 32, row,
+    col % 32]; rows from ``rows`` on are never written, and what is read of them goes nowhere),
+    for the product that takes them next: it then asks the L2 for one piece of rows x 64 bytes
+    per load where rows laid out one after the other give it that many pieces. Made by
+    ``decode_attention``, ``linear_swiglu`` and ``add_rmsnorm`` where the caller allows it
+    (``by_tile``: the caller hands the result to ``linear``, ``linear_swiglu`` or
+    ``linear_add_norm`` and nowhere else), taken by those."""
     __slots__ = ("data", "rows", "dim")
 
     def __init__(self, data, rows, dim):
@@ -210,6 +213,10 @@ class HipKernels:
         # weights, 64 rows: down 17 against 28 us, O 10 against 11 us; 32 rows: 14 against 21 us
         # and 7.5 against 9 us). 0 rows: never.
         self.parts_rows, self.parts_min_k = 64, 2048
+        # Products of 17 to ``stream_rows`` rows whose consumer wants whole sums (QKV, gate / up
+        # with its activation, the output head): K outermost, a workgroup's sums in registers
+        # and x read once per workgroup, instead of the library's product. 0 rows: never.
+        self.stream_rows, self.stream_min_items = 64, 256
         # steps of at most 16 rows: a branch's last projection adds to the residual and leaves
         # the norm's factor to the next product (linear_add_norm) instead of a norm kernel
         self.fuse_norms = True
@@ -282,9 +289,11 @@ class HipKernels:
                                       c_int(_DTYPE_CODE[table.dtype]), self._stream()), "embedding")
         return out
 
-    def add_rmsnorm(self, residual, delta, weight, eps, rows=None):
+    def add_rmsnorm(self, residual, delta, weight, eps, rows=None, by_tile=False):
         """``delta``: None, a [N, d] tensor of the compute dtype, or float32 partial sums
-        [S, N, d] (what ``linear(..., allow_partial=True)`` returns) that are added in order."""
+        [S, N, d] (what ``linear(..., allow_partial=True)`` returns) that are added in order.
+        ``by_tile``: the caller hands the result to ``linear`` or ``linear_swiglu`` and nowhere
+        else, so 17 to 64 rows may come as a ``RowsByTile``."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
         self._want(weight, "norm weight", torch.float32, (d,))
@@ -297,12 +306,16 @@ class HipKernels:
         if rows is not None:
             self._want(rows, "rows", torch.int32)
         n_out = N if rows is None else rows.numel()
-        out = torch.empty((n_out, d), dtype=self.dtype, device=self.device)
+        tile_rows = 0
+        if (by_tile and self.rows_by_tile and self.dtype == torch.bfloat16 and 16 < n_out <= min(self.stream_rows, 64)
+                and d % 32 == 0 and d <= 8192):
+            tile_rows = (n_out + 15) // 16 * 16
+        out = torch.empty((d // 32, tile_rows, 32) if tile_rows else (n_out, d), dtype=self.dtype, device=self.device)
         _check(self._ew.soc_add_rmsnorm(_ptr(residual), _ptr(whole), _ptr(partials), c_int(n_partials),
                                         c_longlong(N * d), _ptr(weight), _ptr(out), _ptr(rows),
-                                        c_int(n_out), c_int(d), c_float(eps), c_int(self.code),
+                                        c_int(n_out), c_int(d), c_float(eps), c_int(self.code), c_int(tile_rows),
                                         self._stream()), "add_rmsnorm")
-        return out
+        return RowsByTile(out, n_out, d) if tile_rows else out
 
     def rmsnorm(self, x, weight, eps):
         dim = x.shape[-1]
@@ -333,6 +346,26 @@ class HipKernels:
         owed = x if isinstance(x, NormOwed) else None
         if owed is not None:
             x = owed.x
+        if isinstance(x, RowsByTile):
+            # 17 to 64 rows by tile (from ``add_rmsnorm``): the product with K outermost reads them so
+            M, K = x.shape
+            N = w_gate_up.shape[0]
+            plan = self._stream_plan(M, N, K, swiglu=True) if (
+                interleave == 16 and w_gate_up.dtype == torch.bfloat16 and N % 32 == 0 and self.library_gemm
+                and x.data.shape[1] > 16) else None
+            if plan is not None:
+                self._want(w_gate_up, "weight", None, (N, K))
+                key, xt = (M, N, K, "swiglu", False), x
+                choice = self.product_choice.get(key)
+                if choice is None and self._tuning and not torch.cuda.is_current_stream_capturing():
+                    xr = x.by_rows()
+                    choice = self.product_choice[key] = self._faster(
+                        lambda: self._k_outermost(plan, xt, w_gate_up, torch.empty((M, N // 2), dtype=self.dtype, device=self.device), True),
+                        lambda: self.swiglu(torch.mm(xr, w_gate_up.t()), interleave))
+                if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan, True)):
+                    out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
+                    return self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
+            x = x.by_rows()
         M, K = x.shape
         N = w_gate_up.shape[0]
         if (interleave == 16 and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
@@ -359,6 +392,21 @@ class HipKernels:
                                                           c_int(tiled | (4 if tiled_out else 0)),
                                                           self._stream()), "linear_swiglu")
             return result
+        if (owed is None and interleave == 16 and x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+                and N % 32 == 0 and self.library_gemm):
+            plan = self._stream_plan(M, N, K, swiglu=True)
+            if plan is not None:
+                self._want(x, "x")
+                self._want(w_gate_up, "weight", None, (N, K))
+                key = (M, N, K, "swiglu", False)
+                choice = self.product_choice.get(key)
+                if choice is None and self._tuning and not torch.cuda.is_current_stream_capturing():
+                    choice = self.product_choice[key] = self._faster(
+                        lambda: self._k_outermost(plan, x, w_gate_up, torch.empty((M, N // 2), dtype=self.dtype, device=self.device), True),
+                        lambda: self.swiglu(torch.mm(x, w_gate_up.t()), interleave))
+                if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan, True, by_tile=False)):
+                    out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
+                    return self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
         return self.swiglu(self.linear(owed if owed is not None else x, w_gate_up), interleave)
 
     _SK_SWIGLU, _SK_SCALED = 1, 2
@@ -424,6 +472,51 @@ class HipKernels:
             c_int(plan[0]), c_int(plan[1]), ssq, c_int(tiles), c_int(dim), c_float(eps), c_int(tiled | layout),
             self._stream()),
             f"{what} (sweep) [{M}x{K}] x [{N}x{K}]^T")
+
+    def _stream_plan(self, M, N, K, swiglu=False):
+        """(workgroups, items per workgroup) if this product of 17 to ``stream_rows`` rows takes
+        the form with K outermost."""
+        if not 16 < M <= min(self.stream_rows, 64) or K % 8 or K < 8 or (N + 32) * K * 2 >= 0xfffffff0:
+            return None
+        wgs, per = c_int(0), c_int(0)
+        if not self._gemm.soc_gemm_stream_plan(c_int(M), c_int(N), c_int(K), c_int(1 if swiglu else 0),
+                                               ctypes.byref(wgs), ctypes.byref(per)):
+            return None
+        if wgs.value * per.value < self.stream_min_items:
+            return None
+        return wgs.value, per.value
+
+    @staticmethod
+    def _stream_default(M, N, K, plan, swiglu=False, by_tile=True):
+        """Whether the product with K outermost is taken where no tuning pass has timed it
+        against the library. Measured on an MI355X inside replayed graphs, weights from memory
+        (us, own with x by tile / own with x row by row / library, with the activation kernel
+        where there is one): QKV of 4B-sized layers [6,144 x 2,560] at 32 rows 10.1 / 12.6 / 11.5,
+        at 64 rows 13.3 / 19.4 / 15.7; gate and up [19,456 x 2,560] 23.5 / 24.7 / 27.5 and
+        28.2 / 32.1 / 31.0; 8B-sized [6,144 x 4,096] 14.6 / 17.7 / 15.4 and 19.3 / 26.3 / 18.0,
+        [24,576 x 4,096] 40.3 / 40.6 / 50.0 and 42.9 / 47.4 / 50.6; 32B-sized [51,200 x 5,120],
+        three passes of a workgroup: 106.5 / 118.0 / 102.1 and 118.4 / 153.2 / 112.1; the output
+        head [151,936 x 2,560], seven passes: 160 / 170 / 174 and 199 / 225 / 186. So: up to 32 rows
+        where x comes by tile or the workgroup needs one pass; beyond, one pass with more
+        weights than rows of x per workgroup, or a short K."""
+        tiles = plan[1] * (2 if swiglu else 1)
+        one_pass = tiles <= 6
+        if M <= 32:
+            return one_pass or by_tile
+        return one_pass and by_tile and (16 * tiles >= M or K <= 3072)
+
+    def _k_outermost(self, plan, x, w, out, swiglu=False, what="linear"):
+        (M, K), N = x.shape, w.shape[0]
+        wt, tiled = self._by_tile(w)
+        if isinstance(x, RowsByTile):
+            self._want(x.data, "x by tile", torch.bfloat16, (K // 32, (M + 15) // 16 * 16, 32))
+            x, tiled = x.data, tiled | 2
+        self.forms["stream" + ("_swiglu" if swiglu else "")] += 1
+        _check(self._gemm.soc_gemm_bf16_stream(
+            _ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(_DTYPE_CODE[out.dtype]),
+            c_int(self._SK_SWIGLU if swiglu else 0), c_int(plan[0]), c_int(plan[1]), c_int(tiled), self._stream()),
+            f"{what} (K outermost) [{M}x{K}] x [{N}x{K}]^T")
+        return out
 
     def _parts_plan(self, M, N, K):
         """(parts of K, K per wave, groups) if this product of 17 to 64 rows, whose consumer
@@ -555,16 +648,17 @@ class HipKernels:
 
     def _faster(self, own, library) -> str:
         """Time the two ways of one product and name the faster. Weights come from memory in a
-        decode step (each is read once per step, behind gigabytes of others), so a write over
-        a buffer larger than the caches comes before every timed call."""
+        decode step (each is read once per step, behind gigabytes of others), so a read of
+        a buffer larger than the caches comes before every timed call (a write would leave the
+        memory-side cache full of lines to write back, which the timed call then pays for)."""
         if getattr(self, "_cold", None) is None:
-            self._cold = torch.empty(160 << 20, dtype=torch.float32, device=self.device)     # 640 MB
+            self._cold = torch.zeros(160 << 20, dtype=torch.float32, device=self.device)     # 640 MB
         times = []
         for fn in (library, own):                        # the library first: its own tuning happens at its first call
             fn()
             total = 0.0
             for _ in range(6):
-                self._cold.zero_()
+                self._cold.max()
                 start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 start.record()
                 fn()
@@ -585,6 +679,23 @@ class HipKernels:
         if isinstance(x, NormOwed):
             return self._linear_owed(x, w, out_dtype or self.dtype, n_waves)
         if isinstance(x, RowsByTile):
+            # 17 to 64 rows by tile (from ``add_rmsnorm``): the product with K outermost reads them so
+            if (x.data.shape[1] > 16 and w.dim() == 2 and w.dtype == torch.bfloat16 and x.shape[1] == w.shape[1]
+                    and not allow_partial and self.library_gemm and not (row_tiles or n_waves or k_splits)):
+                (M, K), N = x.shape, w.shape[0]
+                odt = out_dtype or self.dtype
+                plan = self._stream_plan(M, N, K)
+                if plan is not None:
+                    self._want(w, "weight")
+                    key, xt = (M, N, K, odt, False), x
+                    choice = self.product_choice.get(key)
+                    if choice is None and self._tuning and not torch.cuda.is_current_stream_capturing():
+                        xr = x.by_rows()
+                        choice = self.product_choice[key] = self._faster(
+                            lambda: self._k_outermost(plan, xt, w, torch.empty((M, N), dtype=odt, device=self.device)),
+                            lambda: torch.mm(xr, w.t()) if odt == torch.bfloat16 else torch.mm(xr, w.t(), out_dtype=odt))
+                    if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan)):
+                        return self._k_outermost(plan, x, w, torch.empty((M, N), dtype=odt, device=self.device))
             x = x.by_rows()
         self._want(x, "x")
         self._want(w, "weight")
@@ -628,6 +739,19 @@ class HipKernels:
                         lambda: self._sweep_parts(plan, x, w), lambda: torch.mm(x, w.t()))
                 if choice != "library":
                     return self._sweep_parts(plan, x, w)
+        if both_bf16 and not allow_partial and self.library_gemm and not (row_tiles or explicit):
+            # 17 to 64 rows, whole sums: K outermost, unless a tuning pass has timed both and the library won
+            plan = self._stream_plan(M, N, K)
+            if plan is not None:
+                key = (M, N, K, out_dtype, False)
+                choice = self.product_choice.get(key)
+                lib_dtype = out_dtype
+                if choice is None and self._tuning and not torch.cuda.is_current_stream_capturing():
+                    choice = self.product_choice[key] = self._faster(
+                        lambda: self._k_outermost(plan, x, w, torch.empty((M, N), dtype=out_dtype, device=self.device)),
+                        lambda: torch.mm(x, w.t()) if lib_dtype == torch.bfloat16 else torch.mm(x, w.t(), out_dtype=lib_dtype))
+                if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan, by_tile=False)):
+                    return self._k_outermost(plan, x, w, torch.empty((M, N), dtype=out_dtype, device=self.device))
         row_tiles = max(row_tiles, 0)                     # -1: the skinny kernel, whatever the table says
         if own and not explicit and not allow_partial:
             plan = self._sweep_plan(M, N, K)

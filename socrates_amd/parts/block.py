@@ -86,14 +86,23 @@ class PreNormBlock:
             return part.forward(*args, project=lambda y, w: Normed(ops.linear_add_norm(y, w, residual, gain, eps)))
         return part.forward(*args)
 
+    @staticmethod
+    def _norm(norm, consumer, residual, delta):
+        """The sum and the norm before a part. A part that feeds its input to one product of the
+        kernel set and nowhere else (``takes_norm_owed``) leaves the layout of that input to the
+        kernel set, if the norm can write it so (``free_layout``)."""
+        if getattr(norm, "free_layout", False) and getattr(consumer, "takes_norm_owed", False):
+            return norm.add_norm(residual, delta, by_tile=True)
+        return norm.add_norm(residual, delta)
+
     def forward(self, residual, pending, ctx, slot, write=True, nxt=None):
         """residual: fp32 [N, hidden], updated in place. pending: the previous block's
         un-added output, None, or a ``Normed`` (already added, and normed by this block's
         first norm). ``nxt``: the block that runs next, if it is of this arrangement.
         Returns this block's feed-forward output, un-added or as a ``Normed``."""
-        h = pending.rows if isinstance(pending, Normed) else self.norm1.add_norm(residual, pending)
+        h = pending.rows if isinstance(pending, Normed) else self._norm(self.norm1, self.mixer, residual, pending)
         a = self._branch(self.mixer, (h, ctx, slot, write), residual, self.norm2, self.ffn)
-        h = a.rows if isinstance(a, Normed) else self.norm2.add_norm(residual, a)
+        h = a.rows if isinstance(a, Normed) else self._norm(self.norm2, self.ffn, residual, a)
         return self._branch(self.ffn, (h, ctx), residual, getattr(nxt, "norm1", None), getattr(nxt, "mixer", None))
 
 

@@ -19,12 +19,18 @@ class RMSNorm:
         self.spec, self.ops = spec, ops
         self.weight = tensors["weight"]
 
-    def add_norm(self, residual, delta, rows=None):
+    free_layout = True      # add_norm takes ``by_tile``
+
+    def add_norm(self, residual, delta, rows=None, by_tile=False):
         """residual (fp32, [N, dim]) += delta; return norm(residual) in the compute dtype.
 
         With ``rows`` (int32 indices) only those rows are summed and normed, into a
-        new [len(rows), dim] tensor, and ``residual`` is left unchanged.
+        new [len(rows), dim] tensor, and ``residual`` is left unchanged. ``by_tile``: the
+        result goes to one product of the kernel set and nowhere else, so the kernel set may
+        lay it out as that product reads it best.
         """
+        if by_tile and getattr(self.ops, "rows_by_tile", None):
+            return self.ops.add_rmsnorm(residual, delta, self.weight, self.spec.eps, rows, by_tile=True)
         return self.ops.add_rmsnorm(residual, delta, self.weight, self.spec.eps, rows)
 
     def fusable(self):

@@ -319,6 +319,104 @@ def test_products_of_17_to_64_rows_with_k_split_over_sweeping_workgroups(kernel_
         hip.forget_packed()
 
 
+@pytest.mark.parametrize("M,d,N", [(17, 2560, 6144), (40, 2560, 19456), (64, 4096, 6144), (33, 96, 64), (48, 5120, 640)])
+def test_normed_rows_by_tile_into_the_products_with_k_outermost(kernel_sets, M, d, N):
+    """The norm before QKV and before gate / up hands 17 to 64 rows over laid out by tile
+    ([d / 32, rows rounded up to 16, 32]); the products read them so and give the bits they
+    give from rows laid out one after the other."""
+    from socrates_amd.kernels import RowsByTile
+    hip, _ = kernel_sets[torch.bfloat16]
+    res = rnd((M, d), torch.float32, 90)
+    delta = rnd((M, d), torch.bfloat16, 91)
+    gain = (1 + 0.3 * torch.randn(d)).to(DEV)
+    w = rnd((N, d), torch.bfloat16, 92, d ** -0.5)
+    kept = hip.stream_min_items
+    try:
+        hip.stream_min_items = 1
+        hip._stream_default = lambda *a, **k: True
+        r1, r2 = res.clone(), res.clone()
+        tiled = hip.add_rmsnorm(r1, delta, gain, 1e-6, by_tile=True)
+        rows = hip.add_rmsnorm(r2, delta, gain, 1e-6)
+        assert isinstance(tiled, RowsByTile) and tuple(tiled.data.shape) == (d // 32, (M + 15) // 16 * 16, 32)
+        assert torch.equal(tiled.by_rows(), rows) and torch.equal(r1, r2)
+        hip.forms.clear()
+        assert torch.equal(hip.linear(tiled, w), hip.linear(rows, w))
+        assert torch.equal(hip.linear(tiled, w, out_dtype=torch.float32), hip.linear(rows, w, out_dtype=torch.float32))
+        assert torch.equal(hip.linear_swiglu(tiled, w, 16), hip.linear_swiglu(rows, w, 16))
+        assert hip.forms["stream"] == 4 and hip.forms["stream_swiglu"] == 2, dict(hip.forms)
+        # a consumer that wants partial sums, or the library, gets the rows
+        parts = hip.linear(tiled, w, allow_partial=True)
+        close(parts.sum(0) if parts.dim() == 3 else parts, rows.float() @ w.float().T, torch.bfloat16)
+        hip.stream_rows = 0
+        assert not isinstance(hip.add_rmsnorm(res.clone(), delta, gain, 1e-6, by_tile=True), RowsByTile)
+        close(hip.linear(tiled, w), rows.float() @ w.float().T, torch.bfloat16)
+    finally:
+        hip.stream_rows, hip.stream_min_items = 64, kept
+        del hip._stream_default
+    # up to 16 rows, and beyond 64, the norm's output stays as it was
+    for n in (16, 65):
+        assert not isinstance(hip.add_rmsnorm(rnd((n, d), torch.float32, 93), None, gain, 1e-6, by_tile=True), RowsByTile)
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 6144, 2560), (64, 6144, 2560), (32, 19456, 2560), (48, 10240, 5120), (33, 330, 200),
+                                   (64, 24576, 4096), (20, 16, 32), (64, 40000, 2560), (40, 51200, 5120)])
+def test_products_of_17_to_64_rows_with_k_outermost(kernel_sets, M, N, K):
+    """QKV, the output head (float32 out) and gate / up with its activation at 17 to 64 rows:
+    a workgroup keeps the sums of its tiles in registers and walks over K, against float64
+    products; from the weights by tile and row by row (the same bits). Row m of x is scaled by
+    its own factor, so a row that lands in another one's place shows; widths that are no
+    multiple of 16 and K that is no multiple of 32 read the weights' rows; more tiles than one
+    pass of a workgroup holds take several passes."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    x = rnd((M, K), torch.bfloat16, 80) * torch.logspace(-0.5, 0.5, M, device=DEV)[:, None].to(torch.bfloat16)
+    w = rnd((N, K), torch.bfloat16, 81, K ** -0.5)
+    kept = (hip.stream_min_items, hip.pack_min_elements, hip.pack_weights)
+    try:
+        hip.stream_min_items, hip.pack_min_elements = 1, 1
+        hip._stream_default = lambda *a, **k: True          # the form under test, whatever its default rule says
+        assert hip._stream_plan(M, N, K) is not None and hip._stream_plan(16, N, K) is None and hip._stream_plan(65, N, K) is None
+        exact = x.double() @ w.double().T
+        scale = exact.abs().amax(-1, keepdim=True)
+        bound = 2e-5 * max(1, K / 512) ** 0.5
+        got = {}
+        for tiles in (True, False):
+            hip.pack_weights = tiles
+            hip.forget_packed()
+            hip.forms.clear()
+            out32 = hip.linear(x, w, out_dtype=torch.float32)
+            assert hip.forms["stream"] == 1 and out32.dtype == torch.float32, dict(hip.forms)
+            assert ((out32.double() - exact).abs() / scale).max() < bound
+            out16 = hip.linear(x, w)
+            assert torch.equal(out16, out32.to(torch.bfloat16))       # the same sums, rounded once
+            got[tiles] = out32
+            if N % 32 == 0:
+                # rows alternate in blocks of 16: gate rows, then the up rows of the same outputs
+                act = hip.linear_swiglu(x, w, 16)
+                assert hip.forms["stream_swiglu"] == 1, dict(hip.forms)
+                pairs = exact.view(M, N // 32, 2, 16)
+                gate, up = pairs[:, :, 0].reshape(M, N // 2), pairs[:, :, 1].reshape(M, N // 2)
+                want = torch.nn.functional.silu(gate) * up
+                err = (act.double() - want).abs() / want.abs().amax(-1, keepdim=True)
+                assert tuple(act.shape) == (M, N // 2) and err.max() < 6e-3        # one rounding to bfloat16
+                got[tiles, "act"] = act
+        assert torch.equal(got[True], got[False])
+        if N % 32 == 0:
+            assert torch.equal(got[True, "act"], got[False, "act"])
+        # switched off, the same calls go through the library
+        hip.stream_rows = 0
+        try:
+            hip.forms.clear()
+            lib = hip.linear(x, w, out_dtype=torch.float32)
+            assert hip.forms["stream"] == 0 and hip.forms["library"] == 1
+            assert ((lib.double() - exact).abs() / scale).max() < 4 * bound + 1e-4
+        finally:
+            hip.stream_rows = 64
+    finally:
+        hip.stream_min_items, hip.pack_min_elements, hip.pack_weights = kept
+        del hip._stream_default
+        hip.forget_packed()
+
+
 @pytest.mark.parametrize("M,d,K", [(1, 64, 64), (8, 2560, 4096), (16, 80, 224), (5, 2560, 9728), (3, 4096, 96),
                                    (16, 6144, 2560), (9, 48, 32)])
 def test_weights_by_tile_give_the_same_bits(kernel_sets, M, d, K):
