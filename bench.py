@@ -267,6 +267,8 @@ def main(argv=None):
                     help="decode steps with the residual sums and norms in kernels of their own")
     ap.add_argument("--sweep-rows", type=int, default=None,
                     help="rows of a decode step from which its products take the sweep form (0: never)")
+    ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE",
+                    help="set an attribute of the kernel set (a switch or a threshold of HipKernels), e.g. stream_rows=0")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine is "
@@ -292,6 +294,11 @@ def main(argv=None):
                                   block_size=args.block_size)
     V = config.vocab_size
     engine.runner.ops.fuse_norms = not args.no_fused_norms
+    for item_ in args.set:
+        name, _, value = item_.partition("=")
+        if not hasattr(engine.runner.ops, name):
+            ap.error(f"--set {name}: the kernel set has no such attribute")
+        setattr(engine.runner.ops, name, json.loads(value))
     if args.sweep_rows is not None:
         engine.runner.ops.sweep_rows = args.sweep_rows
     if args.split_waves:

@@ -563,7 +563,8 @@ class HipKernels:
         if not (self.dtype == torch.bfloat16 and yx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
                 and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N <= 65536 and self.fuse_norms):
             # (65,536: the sums of squares of a row are summed by one wave per 256 tiles of 16)
-            return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps)
+            # (the rows go to one product and nowhere else, as a NormOwed would: they may lie by tile)
+            return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps, by_tile=True)
         if tiled_y is not None:
             self._want(yx, "y", torch.bfloat16, (K // 32, 16, 32))
             yx_layout = 2

@@ -83,7 +83,11 @@ class DecoderModel:
         if ctx.n_want == 0:
             # The cache is complete after the last block; no logits are asked for.
             return torch.empty((0, self.plan.vocab_size), dtype=torch.float32, device=ops.device)
-        h = self.final_norm.add_norm(residual, pending, rows=ctx.want_index)
+        # (the normed rows go to the head's product and nowhere else: their layout is the kernel set's)
+        if getattr(self.final_norm, "free_layout", False):
+            h = self.final_norm.add_norm(residual, pending, rows=ctx.want_index, by_tile=True)
+        else:
+            h = self.final_norm.add_norm(residual, pending, rows=ctx.want_index)
         return self.head_logits(h)
 
     def head_logits(self, h):

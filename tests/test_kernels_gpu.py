@@ -303,6 +303,8 @@ def test_products_of_17_to_64_rows_with_k_split_over_sweeping_workgroups(kernel_
         gain = (1 + 0.3 * torch.randn(d)).to(DEV)
         r = res.clone()
         out = hip.linear_add_norm(y, w, r, gain, 1e-6)
+        if type(out).__name__ == "RowsByTile":              # what goes to the next product may lie by tile
+            out = out.by_rows()
         h = res.double() + exact
         torch.testing.assert_close(r.double(), h, atol=1e-4 * max(1, K / 512) ** 0.5, rtol=1e-4)
         close(out, h * torch.rsqrt((h ** 2).mean(-1, keepdim=True) + 1e-6) * gain.double(), torch.bfloat16)
@@ -311,6 +313,8 @@ def test_products_of_17_to_64_rows_with_k_split_over_sweeping_workgroups(kernel_
         try:
             assert hip._parts_plan(M, d, K) is None
             lib_out = hip.linear_add_norm(y, w, r2, gain, 1e-6)
+            if type(lib_out).__name__ == "RowsByTile":
+                lib_out = lib_out.by_rows()
         finally:
             hip.parts_rows = 64
         torch.testing.assert_close(out.float(), lib_out.float(), atol=3e-2, rtol=3e-2)

@@ -173,11 +173,14 @@ def test_every_logit_at_the_benchmarks_batch_sizes(wide, wide_batch, dtype, live
     (tests/test_paged_model.py:35-76). 8 and 16 rows: the sweep form of QKV, gate / up and the
     head, the fused attention with key splits that meet in memory, rows handed on by tile, the
     two projections with the residual sum and the next norm in their epilogue, chained over
-    both layers. 24 and 64 rows: library products beside the sweep over parts of K."""
+    both layers. 24 and 64 rows: the products with K outermost (QKV, gate / up with its activation,
+    the head at 24 rows) from rows that the norm lays out by tile, beside the sweep over parts
+    of K and, at 64 rows, the library's product for the head."""
     folder, cfg, w, _ = wide
     prompts, want = wide_batch
     forms = () if dtype == torch.float32 else \
-        ("sweep", "sweep_swiglu", "add_norm", "fused_attention") if live <= 16 else ("parts_of_k", "library", "fused_attention")
+        ("sweep", "sweep_swiglu", "add_norm", "fused_attention") if live <= 16 else \
+        ("parts_of_k", "stream", "stream_swiglu", "fused_attention")
     ops = decode_rows_through_graphs(folder, cfg, w, prompts, want, dtype, live, forms)
     if dtype == torch.bfloat16 and live == 8:
         splits = [int(k.split(":")[1]) for k in ops.forms if k.startswith("fused_attention")]

@@ -503,7 +503,8 @@ class ReluFeedForward:
 def test_a_toy_feed_forward_takes_the_blocks_folded_sums_and_norms():
     """A part defined here opts into the two optional attributes and gets, in short bfloat16
     steps, rows that are still owed their norm and a projection that adds to the residual
-    stream itself; in long steps and with the folding switched off it gets plain tensors. The
+    stream itself; in steps of 17 to 64 rows normed rows laid out by tile; with the folding
+    switched off and in short steps plain tensors. The
     logits agree either way, and with a whole-prompt run."""
     register_part(ReluSpec, ReluFeedForward)
     ops = kernels("hip", torch.bfloat16)
@@ -528,10 +529,11 @@ def test_a_toy_feed_forward_takes_the_blocks_folded_sums_and_norms():
         results[fused] = torch.cat(logits)
         seen[fused] = model.blocks[1].ffn.calls
     ops.fuse_norms = True
-    # the long first step: plain rows in, yet the projection is the block's (it runs product, sum
-    # and norm one after the other); short steps: rows owed their norm
-    assert seen[True][0] == ("Tensor", True) and seen[True][1] == ("NormOwed", True)
-    assert all(kind == "Tensor" for kind, _ in seen[False])
+    # the long first step (20 rows): normed rows in, laid out by tile for the one product they go
+    # to, and the projection is the block's (it runs product, sum and norm one after the other);
+    # short steps: rows owed their norm; with the folding switched off, normed rows throughout
+    assert seen[True][0] == ("RowsByTile", True) and seen[True][1] == ("NormOwed", True)
+    assert seen[False][0][0] == "RowsByTile" and all(kind == "Tensor" for kind, _ in seen[False][1:4])
     torch.testing.assert_close(results[True], results[False], atol=0.1, rtol=5e-2)
     model = DecoderModel(plan, weights, ops)
     cache = CacheManager(cache_needs(plan), 2, 64, 8, 16, ops.dtype, ops.device)
