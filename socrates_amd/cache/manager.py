@@ -171,7 +171,10 @@ class CacheManager:
                 k, v = group.pools[slot_id]
                 self._slots.append(PagedSlot(k, v, group.table, block_size, need.window))
             elif isinstance(need, RowState):
-                state = torch.zeros((max_rows + 1,) + tuple(need.shape), dtype=torch.float32, device=device)
+                kinds = {"float32": torch.float32, "int32": torch.int32, "compute": dtype}
+                if need.dtype not in kinds:
+                    raise ValueError(f"cache slot {slot_id}: a row's state is one of {sorted(kinds)}, not {need.dtype!r}")
+                state = torch.zeros((max_rows + 1,) + tuple(need.shape), dtype=kinds[need.dtype], device=device)
                 self._slots.append(StateSlot(state))
             elif need is None:
                 self._slots.append(None)

@@ -43,7 +43,12 @@ class AttentionSpec:
 
     ``window`` = None: a query at position p sees keys 0..p. ``window`` = w: it
     sees keys max(0, p-w+1)..p. ``qk_norm`` is applied per head before
-    ``position``; either may be None.
+    ``position``; either may be None. Terms that other architectures add to the
+    scores, all off by default: ``distance_slopes`` (one per query head: slope *
+    (key position - query position) is added to the scaled score), ``softcap`` (the
+    score becomes softcap * tanh(score / softcap)), ``sinks`` (a stored tensor
+    ``sinks`` [n_heads]: one more logit per head that takes part in the softmax's
+    sum and has no value).
     """
     hidden: int
     n_heads: int
@@ -53,8 +58,15 @@ class AttentionSpec:
     qk_norm: Optional[RMSNormSpec] = None
     position: Optional[object] = None
     window: Optional[int] = None
+    softcap: Optional[float] = None
+    sinks: bool = False
+    distance_slopes: Optional[Tuple[float, ...]] = None
 
     def __post_init__(self):
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError("softcap must be positive")
+        if self.distance_slopes is not None and len(self.distance_slopes) != self.n_heads:
+            raise ValueError(f"distance_slopes: one per query head ({self.n_heads}), not {len(self.distance_slopes)}")
         if self.n_heads % self.n_kv_heads:
             raise ValueError(f"n_heads {self.n_heads} is not a multiple of n_kv_heads {self.n_kv_heads}")
         if self.head_dim % 16 or not 16 <= self.head_dim <= 256:
@@ -121,8 +133,16 @@ class ModelPlan:
     # (stored name, name of an expected tensor): a checkpoint may also store the first if it
     # holds the very same values as the second (a tied head written out beside the embedding)
     duplicates: Tuple[Tuple[str, str], ...] = field(default=())
+    # What some architectures put between the parts (none of it in the reference's model, so
+    # the defaults leave the step as it is): the embedding's rows times a constant; the logits
+    # times a constant, then logit_softcap * tanh(logits / logit_softcap).
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: Optional[float] = None
 
     def __post_init__(self):
+        if self.logit_softcap is not None and not self.logit_softcap > 0:
+            raise ValueError("logit_softcap must be positive")
         written = set()
         for step in self.order:
             if not 0 <= step.layer < len(self.layers):

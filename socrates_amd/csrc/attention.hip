@@ -52,6 +52,21 @@ __device__ __forceinline__ void merge_partial(float& m, float& l, float (&a)[EPL
     m = mn;
 }
 
+// Terms that an architecture may add to plain softmax attention (none of them in the reference's
+// model; all three are off when the fields are zero / null). They are computed by this kernel
+// only: the MFMA kernels below take plain scores, and their callers send a layer with such a
+// term here.
+//   slopes   [Hq] float32: slopes[h] * (key position - query position) is added to the scaled
+//            score of head h (a bias by distance)
+//   softcap  > 0: the score becomes softcap * tanh(score / softcap) (after the bias)
+//   sinks    [Hq] float32: one more logit per head that takes its share of the softmax and
+//            contributes no value: the sum of weights gains exp(sinks[h] - max)
+struct ScoreTerms {
+    float softcap;
+    const float* sinks;
+    const float* slopes;
+};
+
 template <typename T, int GC>
 __global__ void __launch_bounds__(256)
 paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
@@ -59,7 +74,7 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
                         int table_width, const int* __restrict__ token_rows,
                         const int* __restrict__ positions, T* __restrict__ out,
                         float* __restrict__ part_o, float* __restrict__ part_ml, int Hq, int Hkv,
-                        int BS, float scale, int window, int split_len, int n_splits) {
+                        int BS, float scale, int window, int split_len, int n_splits, ScoreTerms st) {
     const int G = Hq / Hkv;
     const int chunks = (G + GC - 1) / GC;
     const int kvh = blockIdx.x / chunks, g0 = (blockIdx.x % chunks) * GC;
@@ -88,10 +103,11 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
         }
     }
 
-    float m[GC], l[GC], acc[GC][EPL];
+    float m[GC], l[GC], acc[GC][EPL], slope[GC];
 #pragma unroll
     for (int g = 0; g < GC; ++g) {
         m[g] = -INFINITY; l[g] = 0.f;
+        slope[g] = st.slopes && g0 + g < G ? st.slopes[kvh * G + g0 + g] : 0.f;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) acc[g][e] = 0.f;
     }
@@ -118,6 +134,8 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
 #pragma unroll
                     for (int e = 0; e < EPL; ++e) s = fmaf(qr[g][e], kx[u][e], s);
                     s = group16_sum(s);
+                    if (st.slopes) s += slope[g] * (float)(base + 16 * u - p);
+                    if (st.softcap > 0.f) s = st.softcap * tanhf(s / st.softcap);
                     const float mn = fmaxf(m[g], s);
                     const float alpha = soc_exp<T>(m[g] - mn);      // 0 on the first key (m = -inf)
                     const float w = soc_exp<T>(s - mn);
@@ -171,6 +189,11 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
         }
         const int h = kvh * G + g0 + g;
         if (n_splits == 1) {
+            if (st.sinks) {                                  // the sink's share of the weights, no value
+                const float sk = st.sinks[h], M2 = fmaxf(M, sk), sc = soc_exp<T>(M - M2);
+                L = L * sc + soc_exp<T>(sk - M2);
+                A *= sc;
+            }
             out[((size_t)n * Hq + h) * D + e] = from_float<T>(A / L);
         } else {
             const size_t pi = ((size_t)n * Hq + h) * n_splits + split;
@@ -184,15 +207,15 @@ template <typename T>
 __global__ void paged_attn_reduce_kernel(const float* __restrict__ part_o,
                                          const float* __restrict__ part_ml,
                                          const int* __restrict__ positions, T* __restrict__ out,
-                                         int Hq, int window, int split_len, int n_splits) {
+                                         int Hq, int window, int split_len, int n_splits, ScoreTerms st) {
     const int h = blockIdx.x, n = blockIdx.y;
     const int p = positions[n];
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
     const int np = min(n_splits, (p + 1 - lo + split_len - 1) / split_len);
     const size_t base = ((size_t)n * Hq + h) * n_splits;
-    float M = -INFINITY;
+    float M = st.sinks ? st.sinks[h] : -INFINITY;
     for (int s = 0; s < np; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
-    float L = 0.f;
+    float L = st.sinks ? soc_exp<T>(st.sinks[h] - M) : 0.f;
     for (int s = 0; s < np; ++s) L += part_ml[(base + s) * 2 + 1] * soc_exp<T>(part_ml[(base + s) * 2] - M);
     for (int e = threadIdx.x; e < D; e += blockDim.x) {
         float A = 0.f;
@@ -206,16 +229,16 @@ template <typename T, int GC>
 static int launch_token(const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                         int table_width, const int* token_rows, const int* positions, void* out,
                         float* part_o, float* part_ml, int N, int Hq, int Hkv, int BS, float scale,
-                        int window, int split_len, int n_splits, hipStream_t stream) {
+                        int window, int split_len, int n_splits, ScoreTerms st, hipStream_t stream) {
     const int G = Hq / Hkv, chunks = (G + GC - 1) / GC;
     hipLaunchKernelGGL((paged_attn_token_kernel<T, GC>), dim3(Hkv * chunks, N, n_splits), dim3(256), 0,
                        stream, (const T*)q, (const T*)k_pool, (const T*)v_pool, block_table,
                        table_width, token_rows, positions, (T*)out, part_o, part_ml, Hq, Hkv, BS,
-                       scale, window, split_len, n_splits);
+                       scale, window, split_len, n_splits, st);
     int err = soc_last_error();
     if (err || n_splits == 1) return err;
     hipLaunchKernelGGL(paged_attn_reduce_kernel<T>, dim3(Hq, N), dim3(64), 0, stream, part_o, part_ml,
-                       positions, (T*)out, Hq, window, split_len, n_splits);
+                       positions, (T*)out, Hq, window, split_len, n_splits, st);
     return soc_last_error();
 }
 
@@ -224,9 +247,9 @@ static int dispatch_token(int G, const void* q, const void* k_pool, const void* 
                           const int* block_table, int table_width, const int* token_rows,
                           const int* positions, void* out, float* part_o, float* part_ml, int N,
                           int Hq, int Hkv, int BS, float scale, int window, int split_len,
-                          int n_splits, hipStream_t stream) {
+                          int n_splits, ScoreTerms st, hipStream_t stream) {
 #define SOC_ARGS q, k_pool, v_pool, block_table, table_width, token_rows, positions, out, part_o, \
-                 part_ml, N, Hq, Hkv, BS, scale, window, split_len, n_splits, stream
+                 part_ml, N, Hq, Hkv, BS, scale, window, split_len, n_splits, st, stream
     if (G == 1) return launch_token<T, 1>(SOC_ARGS);
     if (G == 2) return launch_token<T, 2>(SOC_ARGS);
     if (G <= 4) return launch_token<T, 4>(SOC_ARGS);
@@ -237,25 +260,28 @@ static int dispatch_token(int G, const void* q, const void* k_pool, const void* 
 
 // q [N, Hq, D]; pools [pages, Hkv, BS, D]; out [N, Hq, D]. window <= 0: no window.
 // n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml [N, Hq, n_splits, 2] (float32);
-// split s covers keys lo + s * split_len .. of each token.
+// split s covers keys lo + s * split_len .. of each token. softcap (0: none), sinks and slopes
+// ([Hq] float32 each, or null): see ScoreTerms. Any scale, also none or a negative one.
 SOC_EXPORT int soc_paged_attention_tokens(const void* q, const void* k_pool, const void* v_pool,
                                           const int* block_table, int table_width,
                                           const int* token_rows, const int* positions, void* out,
                                           float* part_o, float* part_ml, int N, int Hq, int Hkv,
                                           int BS, float scale, int window, int split_len,
-                                          int n_splits, int dtype, hipStream_t stream) {
+                                          int n_splits, int dtype, float softcap, const float* sinks,
+                                          const float* slopes, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 1) return (int)hipErrorInvalidValue;
+    if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 1 || softcap < 0.f) return (int)hipErrorInvalidValue;
+    const ScoreTerms st{softcap, sinks, slopes};
     if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
     if (N > 65535 || n_splits > 65535) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
     if (dtype == 0)
         return dispatch_token<float>(G, q, k_pool, v_pool, block_table, table_width, token_rows,
                                      positions, out, part_o, part_ml, N, Hq, Hkv, BS, scale, window,
-                                     split_len, n_splits, stream);
+                                     split_len, n_splits, st, stream);
     return dispatch_token<bf16>(G, q, k_pool, v_pool, block_table, table_width, token_rows, positions,
                                 out, part_o, part_ml, N, Hq, Hkv, BS, scale, window, split_len,
-                                n_splits, stream);
+                                n_splits, st, stream);
 }
 
 

@@ -290,6 +290,26 @@ __global__ void swiglu_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __r
     }
 }
 
+// x = scale * x, then (cap > 0) x = cap * tanh(x / cap), in place on float32: what an
+// architecture may ask for behind the embedding (a multiplier) and on the logits (a
+// multiplier, a soft cap). The reference's model has neither.
+__global__ void scale_softcap_kernel(float* __restrict__ x, size_t n, float scale, float cap) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        float v = x[i] * scale;
+        if (cap > 0.f) v = cap * tanhf(v / cap);
+        x[i] = v;
+    }
+}
+
+SOC_EXPORT int soc_scale_softcap(float* x, long long n, float scale, float cap, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if (cap < 0.f) return (int)hipErrorInvalidValue;
+    size_t blocks = ((size_t)n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL(scale_softcap_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, (size_t)n, scale, cap);
+    return soc_last_error();
+}
+
 SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int interleave, int dtype,
                           hipStream_t stream) {
     const size_t total = (size_t)N * ff;

@@ -9,8 +9,10 @@ places. Generation, trace replay and the benchmark all go through it.
 
 from __future__ import annotations
 
+import dataclasses
 from typing import List
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager
@@ -18,6 +20,36 @@ from ..config import load_config
 from ..parts import DecoderModel, cache_needs, expected_tensors
 from ..weights import load_weights
 from .batch import NoHostView, PinnedUploader, StepContext, StepEntry, build_context
+
+
+class _CapturedStep:
+    """A decode step of one width and context bucket, ready to be run again: graphs of the
+    pieces that can be captured, in order, and between them the blocks that cannot, run as
+    they come, each with its output copied to the place the next graph reads."""
+
+    def __init__(self, model, cache, ctx_seen):
+        self.model, self.cache, self.ctx_seen = model, cache, ctx_seen
+        self.pieces = []
+
+    def graph(self, graph):
+        self.pieces.append(graph)
+
+    def eager(self, residual, pending, lo, hi):
+        out = self.model.run(residual, pending, self.ctx_seen, self.cache, lo, hi, last_chains=False)
+        if not isinstance(out, torch.Tensor):
+            raise TypeError("a block that cannot be captured has to return a tensor")
+        fixed = torch.empty_like(out)
+        fixed.copy_(out)
+        self.pieces.append((residual, pending, lo, hi, fixed))
+        return fixed
+
+    def replay(self):
+        for piece in self.pieces:
+            if isinstance(piece, tuple):
+                residual, pending, lo, hi, fixed = piece
+                fixed.copy_(self.model.run(residual, pending, self.ctx_seen, self.cache, lo, hi, last_chains=False))
+            else:
+                piece.replay()
 
 
 class ModelRunner:
@@ -91,14 +123,21 @@ class ModelRunner:
 
     def enable_graphs(self, max_width: int) -> None:
         """From now on steps in which every request brings one token are replayed from HIP
-        graphs, up to ``max_width`` requests. A model with a part that cannot be captured
-        (``capturable = False``: it reads the host's view of the batch or waits for the
-        device) keeps all its steps eager; ``graphs_refused`` then says so."""
+        graphs, up to ``max_width`` requests. A part that cannot be captured (``capturable =
+        False``: it reads the host's view of the batch or waits for the device) is run as it
+        comes, between the graphs of the blocks before and after it; a model with no block
+        that can be captured, or whose final norm cannot, keeps all its steps eager, and
+        ``graphs_refused`` then says so."""
         if self.ops.device.type != "cuda":
             return                       # a stand-in kernel set on the CPU has nothing to capture
         if not getattr(self.model, "capturable", True):
-            self.graphs_refused = "a part of the model declares capturable = False"
-            return
+            segments = self.model.segments() if hasattr(self.model, "segments") else []
+            if not getattr(self.model.final_norm, "capturable", True):
+                self.graphs_refused = "the final norm declares capturable = False"
+                return
+            if not any(cap for cap, _, _ in segments):
+                self.graphs_refused = "no block of the model can be captured (capturable = False)"
+                return
         self._graphs = {}
         self._graph_max = max_width
         self._graph_pool = torch.cuda.graph_pool_handle()
@@ -169,23 +208,54 @@ class ModelRunner:
         inputs = torch.zeros((4, width), dtype=torch.int32, device=dev)
         inputs[2].fill_(self.cache.null_row)
         staging = torch.zeros((4, width), dtype=torch.int32).pin_memory()
+        host = staging.numpy()
+        host[2] = self.cache.null_row
         arange = torch.arange(width + 1, dtype=torch.int32, device=dev)
         ctx = StepContext(
             n_tokens=width, n_seqs=width, n_want=width, token_ids=inputs[0], positions=inputs[1],
             token_rows=inputs[2], seq_rows=inputs[2], seq_qstart=arange, seq_ctx=inputs[3],
             want_index=arange[:width], max_q_len=1, max_ctx_len=context, host=NoHostView())
+        model, cache = self.model, self.cache
+        segments = model.segments() if not getattr(model, "capturable", True) else [(True, 0, len(model.plan.order))]
+        # What a part that is run as it comes sees of the step: the same device tensors, and
+        # the host's arrays of the staging buffer, which is filled before every replay.
+        seen = dataclasses.replace(ctx, host={
+            "positions": host[1], "token_rows": host[2], "seq_rows": host[2],
+            "seq_qstart": np.arange(width + 1, dtype=np.int32), "seq_ctx": host[3]}) if len(segments) > 1 else ctx
         stream = torch.cuda.Stream(device=dev)
         stream.wait_stream(torch.cuda.current_stream(dev))
         with torch.cuda.stream(stream):
-            self.model.forward(ctx, self.cache)          # warm up outside the capture
+            model.forward(seen, cache)                   # warm up outside the capture
         torch.cuda.current_stream(dev).wait_stream(stream)
         torch.cuda.synchronize(dev)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, pool=self._graph_pool, stream=stream):
-            logits = self.model.forward(ctx, self.cache)
-        # The graph holds raw addresses: every tensor it reads (the inputs, and ``arange``
-        # through ctx) has to live as long as the graph, so ctx is kept beside it.
-        return graph, inputs, staging, logits, ctx
+        # The graphs hold raw addresses: every tensor they read (the inputs, ``arange`` through
+        # ctx, what one piece hands to the next) lives as long as the record, which keeps it.
+        step = _CapturedStep(model, cache, seen)
+        residual = pending = logits = None
+        for n, (capturable, lo, hi) in enumerate(segments):
+            first, last = n == 0, n == len(segments) - 1
+            if capturable or first:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self._graph_pool, stream=stream):
+                    if first:
+                        residual, pending = model.begin(ctx)
+                    if capturable:
+                        pending = model.run(residual, pending, ctx, cache, lo, hi)
+                        if last:
+                            logits = model.finish(residual, pending, ctx)
+                step.graph(graph)
+                if len(segments) > 1:
+                    graph.replay()                       # what a block that runs as it comes sees now is a step's values
+            if not capturable:
+                # as it comes, now and at every replay; what it leaves goes to a fixed place
+                # for the graph behind it
+                pending = step.eager(residual, pending, lo, hi)
+                if last:
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, pool=self._graph_pool, stream=stream):
+                        logits = model.finish(residual, pending, ctx)
+                    step.graph(graph)
+        return step, inputs, staging, logits, ctx
 
     def _step_captured(self, entries: List[StepEntry], borrow: bool, fed: torch.Tensor = None) -> torch.Tensor:
         cache = self.cache

@@ -43,6 +43,7 @@ _EW_SIGNATURES = {
     "soc_add_rmsnorm": [P, P, P, I, c_longlong, P, P, P, I, I, F, I, I, P],
     "soc_rmsnorm": [P, P, P, I, I, F, I, P],
     "soc_swiglu": [P, P, I, I, I, I, P],
+    "soc_scale_softcap": [P, c_longlong, F, F, P],
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
     "soc_rope": [P, P, P, I, I, I, I, I, P],
     "soc_kv_write": [P] * 5 + [I, P, P, I, I, I, I, I, P],
@@ -64,7 +65,7 @@ _GEMM_SIGNATURES = {
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
-    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P],
+    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, P],
     "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, I, P],
@@ -325,6 +326,16 @@ class HipKernels:
         _check(self._ew.soc_rmsnorm(_ptr(x), _ptr(weight), _ptr(out), c_int(x.numel() // dim), c_int(dim),
                                     c_float(eps), c_int(self.code), self._stream()), "rmsnorm")
         return out
+
+    def scale_softcap_(self, x, scale=1.0, softcap=None):
+        """In place on float32 ``x``: x * scale, then softcap * tanh(x / softcap) if a soft cap
+        is given."""
+        self._want(x, "x", torch.float32)
+        if softcap is not None and not softcap > 0:
+            raise KernelError("a soft cap is positive")
+        _check(self._ew.soc_scale_softcap(_ptr(x), c_longlong(x.numel()), c_float(scale), c_float(softcap or 0.0),
+                                          self._stream()), "scale_softcap")
+        return x
 
     def swiglu(self, gate_up, interleave=0):
         """silu(gate) * up from a [N, 2 ff] tensor holding [gate | up] (interleave 0) or gate and
@@ -1018,7 +1029,7 @@ class HipKernels:
         return out
 
     def decode_attention(self, qkv, Hq, Hkv, D, q_gain, k_gain, eps, rope_table, slot, ctx, scale,
-                         window=None, write=True, by_tile=False):
+                         window=None, write=True, by_tile=False, terms=None):
         """A decode step's attention straight from the QKV product's rows: per-head norm,
         rotation, the write of the new key and value, and the attention over the pages in one
         kernel. ``qkv`` [N, (Hq + 2 Hkv) D] (with ``write``) or [N, Hq D]. Returns [N, Hq D],
@@ -1028,6 +1039,8 @@ class HipKernels:
         head: a lane's slices of a head then hold both partners of every rotated pair).
         ``by_tile``: the caller hands the result to ``linear_add_norm`` or ``linear`` only, so up
         to 16 rows may come as a ``RowsByTile``."""
+        if terms is not None or not scale > 0:
+            return None                 # scores with further terms, or an unusual scale: the plain kernel's
         if not (self.fuse_rope and self.dtype == torch.bfloat16 and self.attention_mfma
                 and getattr(ctx, "max_q_len", 0) == 1 and D % 32 == 0 and 32 <= D <= 256
                 and (rope_table is None or D % 64 == 0) and slot is not None):
@@ -1078,8 +1091,14 @@ class HipKernels:
             c_int(1 if tiled else 0), self._stream()), "decode_attention")
         return RowsByTile(out, N, Hq * D) if tiled else out
 
-    def paged_attention(self, q, slot, ctx, scale, window=None):
-        """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]."""
+    def paged_attention(self, q, slot, ctx, scale, window=None, terms=None):
+        """q [N, Hq, D] against the pages of each token's row; returns [N, Hq * D]. ``terms``:
+        what an architecture adds to plain softmax attention, a dict with any of ``softcap``
+        (float: scores become softcap * tanh(scores / softcap)), ``sinks`` (float32 [Hq]: one
+        more logit per head in the softmax's sum, with no value) and ``slopes`` (float32 [Hq]:
+        slope * (key position - query position) added to the scaled scores). Such a layer,
+        and one whose scale is not positive, goes to the kernel that computes scores on the
+        vector units, in either dtype; the MFMA kernels take plain scores only."""
         N, Hq, D = q.shape
         self._want(q, "q", self.dtype)
         Hkv = slot.k.shape[1]
@@ -1092,7 +1111,19 @@ class HipKernels:
         out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
         w = int(window) if window else 0
         G = Hq // Hkv
-        if self.dtype == torch.bfloat16 and self.attention_mfma:
+        softcap, sinks, slopes = 0.0, None, None
+        if terms:
+            if set(terms) - {"softcap", "sinks", "slopes"}:
+                raise KernelError(f"attention: unknown score terms {sorted(set(terms) - {'softcap', 'sinks', 'slopes'})}")
+            softcap = float(terms.get("softcap") or 0.0)
+            sinks, slopes = terms.get("sinks"), terms.get("slopes")
+            if softcap < 0:
+                raise KernelError("attention: a soft cap is positive")
+            for name, t in (("sinks", sinks), ("slopes", slopes)):
+                if t is not None:
+                    self._want(t, name, torch.float32, (Hq,))
+        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0
+        if self.dtype == torch.bfloat16 and self.attention_mfma and plain:
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
             if N > 65535:
@@ -1176,7 +1207,8 @@ class HipKernels:
                 _ptr(part_o[lo:lo + n]) if part_o is not None else None,
                 _ptr(part_ml[lo:lo + n]) if part_ml is not None else None,
                 c_int(n), c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w),
-                c_int(split_len), c_int(n_splits), c_int(self.code), self._stream()), "paged_attention")
+                c_int(split_len), c_int(n_splits), c_int(self.code), c_float(softcap), _ptr(sinks), _ptr(slopes),
+                self._stream()), "paged_attention")
         return out
 
     # -- sampling ------------------------------------------------------------------------------

@@ -29,6 +29,8 @@ class PagedAttention:
         if spec.qk_norm is not None:
             t["q_norm.weight"] = TensorDecl((D,), "vector")
             t["k_norm.weight"] = TensorDecl((D,), "vector")
+        if spec.sinks:
+            t["sinks"] = TensorDecl((spec.n_heads,), "vector")
         return t
 
     @staticmethod
@@ -49,6 +51,15 @@ class PagedAttention:
         self.position = (build_part(spec.position, {}, ops)
                          if spec.position is not None else None)
         self.capturable = getattr(self.position, "capturable", True)
+        # terms beyond plain softmax attention, for the kernel set (None: plain)
+        terms = {}
+        if spec.softcap is not None:
+            terms["softcap"] = float(spec.softcap)
+        if spec.sinks:
+            terms["sinks"] = tensors["sinks"]
+        if spec.distance_slopes is not None:
+            terms["slopes"] = torch.tensor(spec.distance_slopes, dtype=torch.float32, device=ops.device)
+        self.terms = terms or None
         self._free_layout = {"by_tile": True} if getattr(ops, "rows_by_tile", None) is not None else {}
 
     def reserve(self, n_positions):
@@ -72,7 +83,7 @@ class PagedAttention:
         rot = self.position.rotary() if hasattr(self.position, "rotary") else None
         o = None
         if ((self.position is None or rot is not None) and hasattr(ops, "decode_attention")
-                and ctx.max_q_len == 1):
+                and ctx.max_q_len == 1 and self.terms is None):
             # a decode step: norm, position encoding, cache write and attention in one kernel
             table = self.position.table(ctx.max_ctx_len) if hasattr(self.position, "table") else None
             if self.position is None or table is not None:
@@ -93,7 +104,8 @@ class PagedAttention:
             if write:
                 ops.kv_write(k, v, ctx.positions, ctx.token_rows, slot)
         if o is None:
-            o = ops.paged_attention(q, slot, ctx, s.scale, s.window)
+            o = (ops.paged_attention(q, slot, ctx, s.scale, s.window) if self.terms is None
+                 else ops.paged_attention(q, slot, ctx, s.scale, s.window, terms=self.terms))
         if project is not None:
             return project(o, self.w_o)
         # the block's next norm adds this output to the residual: partial sums are welcome

@@ -59,8 +59,10 @@ class PagedKV:
 
 @dataclass(frozen=True)
 class RowState:
-    """A mixer that keeps a state of fixed size per request (float32)."""
+    """A mixer that keeps a state of fixed size per request: ``shape`` elements of ``dtype``
+    ("float32", "int32", or "compute": the model's compute dtype), zero when a row opens."""
     shape: Tuple[int, ...]
+    dtype: str = "float32"
 
 
 def register_part(spec_type, impl) -> None:

@@ -750,6 +750,39 @@ def test_workgroups_that_meet_in_memory_give_the_same_bits_every_time(kernel_set
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,bs", [(8, 2, 64, 16), (6, 3, 48, 4), (32, 8, 128, 16)])
+def test_attention_with_further_score_terms(kernel_sets, dtype, Hq, Hkv, D, bs):
+    """A bias by distance, a soft cap and a sink logit per head, one at a time and together,
+    with and without key splits and a window, decoded tokens and a prompt portion, in both
+    dtypes (such a layer goes to the kernel that computes scores on the vector units), against
+    the torch stand-in's formulas on the same pages; also a scale that is not positive."""
+    hip, ref = kernel_sets[dtype]
+    lens = [1, 17, 70, 300]
+    slot, _ = make_paged_case(lens, Hq, Hkv, D, bs, dtype, seed=D + 7)
+    rows = [0, 1] + [2] * 20 + [3]
+    pos = [0, 16] + list(range(50, 70)) + [299]
+    q = rnd((len(rows), Hq, D), dtype, 31)
+    ctx = ctx_for(rows, pos)
+    sinks = torch.linspace(-2, 3, Hq, device=DEV)
+    slopes = -torch.logspace(-3, -0.5, Hq, device=DEV)
+    cases = [dict(softcap=4.0), dict(sinks=sinks), dict(slopes=slopes), dict(softcap=2.5, sinks=sinks, slopes=slopes)]
+    for terms in cases:
+        for window in (None, 33):
+            want = ref.paged_attention(q, slot, ctx, 0.3, window, terms=terms)
+            for splits in (None, (64, 5), (1 << 30, 1)):
+                hip.attention_splits = splits
+                got = hip.paged_attention(q, slot, ctx, 0.3, window, terms=terms)
+                close(got.cpu(), want.cpu(), dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+            hip.attention_splits = None
+        plain_ = ref.paged_attention(q, slot, ctx, 0.3, None)
+        assert (ref.paged_attention(q, slot, ctx, 0.3, None, terms=terms).float() - plain_.float()).abs().max() > 0.02
+    got = hip.paged_attention(q, slot, ctx, -0.2)              # the MFMA kernels want a positive scale
+    close(got.cpu(), ref.paged_attention(q, slot, ctx, -0.2, None).cpu(), dtype, atol=3e-5 if dtype == torch.float32 else 2e-2)
+    with pytest.raises(Exception, match="unknown score terms"):
+        hip.paged_attention(q, slot, ctx, 0.3, terms=dict(alibi=slopes))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_prompt_portions_and_window(kernel_sets, dtype):
     """Tokens of one row at consecutive positions (a portion that starts mid-sequence)
     beside single tokens of other rows, with and without a window."""

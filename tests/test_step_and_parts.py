@@ -304,36 +304,74 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps(kind, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_a_model_with_a_stateful_toy_mixer_generates_through_the_engine(dtype):
     """``Engine(compile=True)``, the default, with a model one of whose parts cannot be
-    captured: the runner keeps every step eager (and says why), generation works, tokens are
-    those of ``compile=False``, and a model of capturable parts beside it does get its graphs.
-    A captured step's context has no host view, and says so when asked."""
+    captured: the runner captures the blocks before and after it and runs that block as it
+    comes, with the host's view of the batch (steps are queued ahead as for any model);
+    tokens are those of ``compile=False``. A model none of whose blocks can be captured keeps
+    every step eager and says why. A captured step's context has no host view, and says so
+    when asked."""
     from socrates_amd.engine import Engine, NoHostView
     from socrates_amd.kernels import HipKernels
     register_part(DecaySpec, DecayMixer)
     ops = HipKernels(dtype, "cuda:0")
     hidden = 32
-    toy = BlockSpec(DecaySpec(hidden, 0.9), SwiGLUSpec(hidden, 40), RMSNormSpec(hidden, 1e-5),
-                    RMSNormSpec(hidden, 1e-5), prefix="model.layers.1.",
-                    names=(("norm1", "n1"), ("mixer", "decay"), ("norm2", "n2"), ("ffn", "mlp")))
+
+    def toy(i):
+        return BlockSpec(DecaySpec(hidden, 0.9), SwiGLUSpec(hidden, 40), RMSNormSpec(hidden, 1e-5),
+                         RMSNormSpec(hidden, 1e-5), prefix=f"model.layers.{i}.",
+                         names=(("norm1", "n1"), ("mixer", "decay"), ("norm2", "n2"), ("ffn", "mlp")))
     prompts = random_prompts([9, 3, 14], 50, seed=2)
     outs = {}
-    for label, layers, compile_ in (("toy", [qwen_like_block(0), toy], True), ("toy-eager", [qwen_like_block(0), toy], False),
+    mixed = [qwen_like_block(0), toy(1), qwen_like_block(2), qwen_like_block(3), toy(4)]
+    for label, layers, compile_ in (("toy", mixed, True), ("toy-eager", mixed, False),
+                                    ("toy-first", [toy(0), qwen_like_block(1)], True),
+                                    ("toy-first-eager", [toy(0), qwen_like_block(1)], False),
+                                    ("all-toy", [toy(0), toy(1)], True),
                                     ("plain", [qwen_like_block(0), qwen_like_block(1)], True)):
-        plan = plan_with(layers, [RunStep(0, 0), RunStep(1, 1)], hidden)
+        plan = plan_with(layers, [RunStep(i, i) for i in range(len(layers))], hidden)
         weights = random_tensors(expected_tensors(plan), seed=3, dtype=dtype, device="cuda:0", std=0.2, gain_std=0.1)
         model = DecoderModel(plan, weights, ops)
         cache = CacheManager(cache_needs(plan), 4, 64, 8, 32, dtype, "cuda:0")
         engine = Engine(ModelRunner(model, cache), max_batch=4, max_len=64, max_new_tokens=10, compile=compile_)
         outs[label] = engine.generate(prompts, max_new_tokens=10)
         if label == "toy":
-            assert not model.capturable and engine.runner._graphs is None
-            assert "capturable" in engine.runner.graphs_refused
+            assert not model.capturable and engine.runner._graphs and engine.runner.graphs_refused is None
+            assert model.segments() == [(True, 0, 1), (False, 1, 2), (True, 2, 4), (False, 4, 5)]
+            step = next(iter(engine.runner._graphs.values()))[0]
+            assert [isinstance(p, tuple) for p in step.pieces] == [False, True, False, True, False]
+            assert engine.n_ahead > 0                        # steps were queued ahead of their tokens
+        elif label == "toy-first":
+            step = next(iter(engine.runner._graphs.values()))[0]
+            assert [isinstance(p, tuple) for p in step.pieces] == [False, True, False]      # the embedding alone, captured
+        elif label == "all-toy":
+            assert engine.runner._graphs is None and "capturable" in engine.runner.graphs_refused
             assert engine.warmup() == 0
         elif label == "plain":
             assert model.capturable and engine.runner._graphs
         assert all(len(o) == 10 for o in outs[label])
         assert not cache.open_rows
-    assert outs["toy"] == outs["toy-eager"]
+    if dtype == torch.float32:
+        assert outs["toy"] == outs["toy-eager"]
+        assert outs["toy-first"] == outs["toy-first-eager"]
+    # the same tokens through both kinds of step, logits compared (in bfloat16 a greedy choice
+    # may flip between two ways of summing, so tokens are compared in float32 only)
+    plan = plan_with(mixed, [RunStep(i, i) for i in range(len(mixed))], hidden)
+    weights = random_tensors(expected_tensors(plan), seed=3, dtype=dtype, device="cuda:0", std=0.2, gain_std=0.1)
+    logits = {}
+    for graphs in (True, False):
+        cache = CacheManager(cache_needs(plan), 4, 64, 8, 32, dtype, "cuda:0")
+        runner = ModelRunner(DecoderModel(plan, weights, ops), cache)
+        if graphs:
+            runner.enable_graphs(4)
+        rows = [cache.open_row() for _ in prompts]
+        runner.step([StepEntry(r, p[:-2], []) for r, p in zip(rows, prompts)])
+        got = [runner.step([StepEntry(r, [p[len(p) - 2 + t]], [0]) for r, p in zip(rows, prompts)]).float().cpu()
+               for t in range(2)]
+        # one request leaves, the others go on: the same graph with a padding row
+        cache.close_row(rows[1])
+        got.append(runner.step([StepEntry(rows[0], [7], [0]), StepEntry(rows[2], [8], [0])]).float().cpu())
+        logits[graphs] = torch.cat(got)
+        assert bool(runner._graphs) == graphs
+    torch.testing.assert_close(logits[True], logits[False], **TOL[dtype])
     with pytest.raises(KeyError, match="capturable = False"):
         NoHostView()["seq_qstart"]
 
@@ -539,3 +577,85 @@ def test_a_toy_feed_forward_takes_the_blocks_folded_sums_and_norms():
     cache = CacheManager(cache_needs(plan), 2, 64, 8, 16, ops.dtype, ops.device)
     whole_run = ModelRunner(model, cache).step([StepEntry(cache.open_row(), tokens, list(range(40)))]).float().cpu()
     torch.testing.assert_close(results[True], whole_run, atol=0.1, rtol=5e-2)
+
+
+def plain_attention_with_terms(q, k, v, scale, slopes=None, softcap=None, sinks=None):
+    """Causal softmax attention written out, with what other architectures add to the scores:
+    slope[h] * (key - query position), then softcap * tanh(. / softcap), and one more logit
+    per head that shares in the softmax's sum and has no value. q [T, Hq, D], k, v [T, Hkv, D]."""
+    T, Hq, D = q.shape
+    G = Hq // k.shape[1]
+    out = torch.empty_like(q)
+    pos = torch.arange(T)
+    for h in range(Hq):
+        s = (q[:, h] @ k[:, h // G].T) * scale
+        if slopes is not None:
+            s = s + slopes[h] * (pos[None, :] - pos[:, None])
+        if softcap is not None:
+            s = softcap * torch.tanh(s / softcap)
+        s = s.masked_fill(pos[None, :] > pos[:, None], float("-inf"))
+        if sinks is not None:
+            s = torch.cat([s, torch.full((T, 1), float(sinks[h]))], dim=-1)
+            a = torch.softmax(s, dim=-1)[:, :-1]
+        else:
+            a = torch.softmax(s, dim=-1)
+        out[:, h] = a @ v[:, h // G]
+    return out
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_a_model_with_further_score_terms_and_scaled_embedding_and_logits(kind, dtype):
+    """What the reference's model does not have and another architecture may: attention with a
+    bias by distance, a soft cap and a sink logit per head (a stored tensor), the embedding
+    times a constant, the logits times a constant under a soft cap. All of it is said in specs
+    and the plan; the attention goes to the kernel that computes scores on the vector units
+    (the MFMA kernels take plain scores) in either dtype, whole prompts and cut ones, decoded
+    tokens too, against the formulas written out here."""
+    import math
+    ops = kernels(kind, dtype)
+    hidden, heads, kv, D, ff, vocab = 32, 4, 2, 16, 48, 50
+    slopes = tuple(-0.5 ** (i + 1) for i in range(heads))
+    att = AttentionSpec(hidden, heads, kv, D, 1.0 / D, RMSNormSpec(D, 1e-6), RopeSpec(D, 1e4),
+                        softcap=5.0, sinks=True, distance_slopes=slopes)
+    plain_att = AttentionSpec(hidden, heads, kv, D, 1.0 / D, RMSNormSpec(D, 1e-6), RopeSpec(D, 1e4))
+    blocks = [BlockSpec(a, SwiGLUSpec(hidden, ff), RMSNormSpec(hidden, 1e-6), RMSNormSpec(hidden, 1e-6),
+                        prefix=f"model.layers.{i}.") for i, a in enumerate((att, plain_att))]
+    plan = ModelPlan(architecture="Toy", vocab_size=vocab, hidden=hidden, layers=tuple(blocks),
+                     order=(RunStep(0, 0), RunStep(1, 1)), final_norm=RMSNormSpec(hidden, 1e-6),
+                     embedding_name="embed.weight", final_norm_prefix="final_norm", head_name=None,
+                     embedding_scale=math.sqrt(hidden), logit_scale=0.5, logit_softcap=3.0)
+    assert "model.layers.0.self_attn.sinks" in expected_tensors(plan)
+    assert "model.layers.1.self_attn.sinks" not in expected_tensors(plan)
+    tokens = random_prompts([37], vocab, seed=6)[0]
+    weights, (whole_run, cut_run) = run_whole_and_cut(plan, ops, tokens, [[37], [9, 1, 1, 20, 1, 5]])
+    w = {n: t.float().cpu() for n, t in weights.items()}
+    # the plain run
+    cfg = dict(num_attention_heads=heads, num_key_value_heads=kv, head_dim=D, rms_norm_eps=1e-6, rope_theta=1e4)
+    x = w["embed.weight"][torch.tensor(tokens)] * math.sqrt(hidden)
+    pos = torch.arange(len(tokens))
+    cos, sin = plain.rope_angles(D, 1e4, pos)
+    for i, terms in enumerate((dict(slopes=slopes, softcap=5.0, sinks=weights["model.layers.0.self_attn.sinks"].float().cpu()), {})):
+        p = f"model.layers.{i}."
+        h = plain.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6)
+        q = (h @ w[p + "self_attn.q_proj.weight"].T).view(-1, heads, D)
+        k = (h @ w[p + "self_attn.k_proj.weight"].T).view(-1, kv, D)
+        v = (h @ w[p + "self_attn.v_proj.weight"].T).view(-1, kv, D)
+        q = plain.apply_rope(plain.rms_norm(q, w[p + "self_attn.q_norm.weight"], 1e-6), cos, sin)
+        k = plain.apply_rope(plain.rms_norm(k, w[p + "self_attn.k_norm.weight"], 1e-6), cos, sin)
+        o = plain_attention_with_terms(q, k, v, 1.0 / D, **terms)
+        x = x + o.reshape(len(tokens), heads * D) @ w[p + "self_attn.o_proj.weight"].T
+        x = x + plain.swiglu_mlp(plain.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6), w, p + "mlp.")
+    logits = plain.rms_norm(x, w["final_norm.weight"], 1e-6) @ w["embed.weight"].T
+    want = 3.0 * torch.tanh(0.5 * logits / 3.0)
+    tol = TOL[dtype]
+    torch.testing.assert_close(whole_run, want, **tol)
+    torch.testing.assert_close(cut_run, want, **tol)
+    # each term matters at these sizes: without it the logits are visibly others
+    for drop in ("slopes", "softcap", "sinks"):
+        terms = dict(slopes=slopes, softcap=5.0, sinks=weights["model.layers.0.self_attn.sinks"].float().cpu())
+        terms.pop(drop)
+        q0 = torch.randn(12, heads, D) * 3
+        k0, v0 = torch.randn(12, kv, D) * 3, torch.randn(12, kv, D)
+        full = plain_attention_with_terms(q0, k0, v0, 0.25, slopes=slopes, softcap=5.0,
+                                          sinks=weights["model.layers.0.self_attn.sinks"].float().cpu())
+        assert (plain_attention_with_terms(q0, k0, v0, 0.25, **terms) - full).abs().max() > 1e-2, drop

@@ -55,6 +55,12 @@ class TorchKernels:
     def rmsnorm(self, x, weight, eps):
         return self._norm(x, weight, eps).to(x.dtype)
 
+    def scale_softcap_(self, x, scale=1.0, softcap=None):
+        x.mul_(scale)
+        if softcap is not None:
+            x.copy_(softcap * torch.tanh(x / softcap))
+        return x
+
     def swiglu(self, gate_up, interleave=0):
         ff = gate_up.shape[-1] // 2
         if interleave:
@@ -119,8 +125,11 @@ class TorchKernels:
             self.kv_write(k, v, positions, token_rows, slot)
         return q.to(self.dtype).contiguous()
 
-    def paged_attention(self, q, slot, ctx, scale, window):
-        """Token by token: gather the row's keys 0..p through the table, mask the window."""
+    def paged_attention(self, q, slot, ctx, scale, window, terms=None):
+        """Token by token: gather the row's keys 0..p through the table, mask the window.
+        ``terms``: a bias by distance (``slopes`` [Hq]), a soft cap of the scores, one more
+        logit per head in the softmax's sum (``sinks`` [Hq])."""
+        terms = terms or {}
         N, Hq, D = q.shape
         Hkv, bs = slot.k.shape[1], slot.block_size
         G = Hq // Hkv
@@ -138,7 +147,16 @@ class TorchKernels:
             v = slot.v[pages, :, offs].to(self.acc)
             qt = q[t].to(self.acc).view(Hkv, G, D)
             s = torch.einsum("hgd,nhd->hgn", qt, k) * scale
-            a = torch.softmax(s, dim=-1)
+            if terms.get("slopes") is not None:
+                dist = torch.as_tensor(idx - p, device=q.device).to(self.acc)
+                s = s + terms["slopes"].to(self.acc).view(Hkv, G, 1) * dist
+            if terms.get("softcap"):
+                s = terms["softcap"] * torch.tanh(s / terms["softcap"])
+            if terms.get("sinks") is not None:
+                s = torch.cat([s, terms["sinks"].to(self.acc).view(Hkv, G, 1)], dim=-1)
+                a = torch.softmax(s, dim=-1)[..., :-1]
+            else:
+                a = torch.softmax(s, dim=-1)
             out[t] = torch.einsum("hgn,nhd->hgd", a, v).reshape(Hq * D).to(self.dtype)
         return out
 
