@@ -320,7 +320,7 @@ template <typename TC, int MT, int RW, int MODE = 0>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, RW, MODE))
 gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, TC* __restrict__ C,
                         float* __restrict__ Cpart, int M, int N, int K, int k_per_split,
-                        int k_per_wave, SkNorm nm, int layout = 0) {
+                        int k_per_wave, SkNorm nm, int layout = 0, int tile_h = 16) {
     constexpr bool SWIGLU = MODE & SK_SWIGLU, SCALED = MODE & SK_SCALED, ADDNORM = MODE & SK_ADDNORM;
     static_assert(!(SCALED || ADDNORM) || (MT == 1 && RW == 1), "the norm forms take one tile of each");
     __shared__ float red[sk_max_waves(MT, RW, MODE) * MT * RW * 256];
@@ -331,7 +331,11 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
     const int k_waves = SWIGLU ? n_waves / 2 : n_waves;        // waves that share one tile's K
-    const int n0 = SWIGLU ? blockIdx.x * 32 + (wave / k_waves) * 16 : blockIdx.x * 16 * RW;
+    // tile_h (the ADDNORM form; 16 elsewhere): weight rows of a workgroup, at most 16. Fewer
+    // than 16 spread a narrow output over more workgroups (2,560 outputs are 160 tiles of 16,
+    // which leave 96 of 256 compute units idle, and 256 tiles of 10); the rows from tile_h on
+    // of the 16 that a product takes are not there.
+    const int n0 = SWIGLU ? blockIdx.x * 32 + (wave / k_waves) * 16 : ADDNORM ? blockIdx.x * tile_h : blockIdx.x * 16 * RW;
     const int li = lane % 16, lk = (lane / 16) * 8;
     const int split_begin = blockIdx.y * k_per_split;
     const int split_end = min(K, split_begin + k_per_split);
@@ -345,7 +349,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     // hands to the next one is then read in pieces of M x 64 bytes instead of M pieces.
     const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED, c_tiled = layout & SK_C_TILED;
     const int w_rs = w_tiled ? 32 : K;              // elements from a row of a tile to the next
-    const int w_ss = w_tiled ? 512 : 32;            // elements from a step of 32 k to the next
+    const int w_ss = w_tiled ? 32 * tile_h : 32;    // elements from a step of 32 k to the next
     const int x_rs = x_tiled ? 32 : K, x_ss = x_tiled ? 512 : 32;
     // Element offsets of this lane's rows (offsets, not pointers: the loads stay global
     // loads); a row outside the matrix is never loaded.
@@ -353,8 +357,8 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     bool w_ok[RW];
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
-        w_ok[r] = n0 + r * 16 + li < N;
-        w_off[r] = w_ok[r] ? (size_t)(n0 + r * 16) * K + (size_t)li * w_rs + lk : (size_t)lk;
+        w_ok[r] = n0 + r * 16 + li < N && li < tile_h;
+        w_off[r] = w_ok[r] ? (size_t)(n0 + r * 16) * K + (size_t)li * w_rs + lk : (size_t)n0 * K + lk;
     }
     // X is read through a buffer descriptor that covers its M rows: a lane whose row lies
     // outside (M = 8 leaves half of the 16 lanes of a tile without one) gets zeros and asks
@@ -378,7 +382,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     float old_h = 0.f, out_gain = 0.f;
     if constexpr (ADDNORM) {
         const int ln = (tid % 256) / 4, e = tid % 4;
-        const int m = min(ln % 16, M - 1), n = min(n0 + 4 * (ln / 16) + e, N - 1);
+        const int m = min(ln % 16, M - 1), n = min(n0 + min(4 * (ln / 16) + e, tile_h - 1), N - 1);
         old_h = nm.residual[(size_t)m * N + n];
         out_gain = nm.gain[n];
     }
@@ -511,7 +515,7 @@ gemm_bf16_skinny_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
         }
         if (tid < 256) {
             float h = 0.f;
-            if (m < M && n < N) {
+            if (m < M && n < N && c < tile_h) {
                 h = old_h + sum;
                 nm.residual[(size_t)m * N + n] = h;
                 nm.x_out[(size_t)m * N + n] = from_float<bf16>(h * out_gain);
@@ -595,16 +599,20 @@ SOC_EXPORT int soc_gemm_bf16_skinny_swiglu(const void* X, const void* W, void* C
 // x_out [M, N] = bf16(residual * gain), ssq_out [M, ceil(N / 16)] are written for the norm of
 // `N` elements that follows; C is then not written. At least one of the two is given.
 // k_splits > 1 (with residual only): K is split over that many workgroups per tile, which meet
-// through split_sums [ceil(N / 16), k_splits, 256] floats (scratch) and split_count
-// [ceil(N / 16)] ints, which must be zero before the call and are zero again after it. Two
+// through split_sums [tiles, k_splits, 256] floats (scratch) and split_count
+// [tiles] ints, which must be zero before the call and are zero again after it. Two
 // launches that may run at the same time need counts of their own.
+// tile_h (with residual; 16 otherwise): weight rows of a workgroup, 1 to 16; tiles = ceil(N /
+// tile_h) workgroups (times k_splits), ssq_out [M, tiles rounded up to 4]; weights by tile then
+// lie [N / tile_h, K / 32, tile_h, 32] (N a multiple of tile_h).
 SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, int M, int N, int K,
                                          int n_waves, const float* ssq_in, int ssq_tiles, int norm_dim,
                                          float eps, float* residual, const float* gain, void* x_out,
                                          float* ssq_out, int k_splits, float* split_sums, int* split_count,
-                                         int layout, hipStream_t stream) {
+                                         int layout, int tile_h, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if ((layout & ~3) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) || ((layout & SK_X_TILED) && K % 32))
+    if (tile_h < 1 || tile_h > 16 || (tile_h != 16 && !residual)) return (int)hipErrorInvalidValue;
+    if ((layout & ~3) || ((layout & SK_W_TILED) && (N % tile_h || K % 32)) || ((layout & SK_X_TILED) && K % 32))
         return (int)hipErrorInvalidValue;
     if (M > 16 || K % 8 || K < 8 || K > (1 << 23)) return (int)hipErrorInvalidValue;
     if (n_waves < 1 || n_waves > SK_MAX_WAVES_SWIGLU) return (int)hipErrorInvalidValue;
@@ -620,10 +628,10 @@ SOC_EXPORT int soc_gemm_bf16_skinny_norm(const void* X, const void* W, void* C, 
     nm.split_sums = split_sums; nm.split_count = split_count;
     nm.ssq_in = ssq_in; nm.ssq_tiles = ssq_tiles; nm.inv_dim = 1.0f / (float)max(norm_dim, 1); nm.eps = eps;
     nm.residual = residual; nm.gain = gain; nm.x_out = (bf16*)x_out; nm.ssq_out = ssq_out;
-    const dim3 grid((N + 15) / 16, k_splits), block(n_waves * 64);
+    const dim3 grid((N + tile_h - 1) / tile_h, k_splits), block(n_waves * 64);
 #define SOC_SKN(MODE_) \
     hipLaunchKernelGGL((gemm_bf16_skinny_kernel<bf16, 1, 1, MODE_>), grid, block, 0, stream, (const bf16*)X, \
-                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, layout)
+                       (const bf16*)W, (bf16*)C, (float*)nullptr, M, N, K, k_per_split, k_per_wave, nm, layout, tile_h)
     if (ssq_in && residual) SOC_SKN(SK_SCALED | SK_ADDNORM);
     else if (residual) SOC_SKN(SK_ADDNORM);
     else SOC_SKN(SK_SCALED);

@@ -55,7 +55,7 @@ _GEMM_SIGNATURES = {
     "soc_gemm_bf16_skinny": [P, P, P, P, I, I, I, I, I, I, I, I, P],
     "soc_gemm_skinny_plan": [I, I, I, I, P, P, P],
     "soc_gemm_bf16_skinny_swiglu": [P, P, P, I, I, I, I, I, P, I, I, F, I, P],
-    "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, I, P, P, I, P],
+    "soc_gemm_bf16_skinny_norm": [P, P, P, I, I, I, I, P, I, I, F, P, P, P, P, I, P, P, I, I, P],
     "soc_gemm_bf16_sweep": [P, P, P, I, I, I, I, I, I, I, P, I, I, F, I, P],
     "soc_gemm_sweep_plan": [I, I, I, P, P],
     "soc_gemm_bf16_sweep_parts": [P, P, P, I, I, I, I, I, I, I, P],
@@ -82,7 +82,7 @@ def _declare(lib, signatures):
 MAX_KEY_SPLITS = 256    # of the MFMA attention: 64 workgroups of four splits meet per task
 
 
-def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, min_keys=64):
+def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, min_keys=64, n_units=256):
     """(split_len, n_splits) for the MFMA attention kernel: enough waves to fill the GPU, no
     split shorter than 64 keys, at most MAX_KEY_SPLITS of them (a longer context gets longer
     splits), one split or a multiple of four (four share a workgroup; some of the last four
@@ -103,6 +103,19 @@ def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, mi
     if n == 1:
         return ((max_keys + 15) // 16 * 16), 1
     n = (n + 3) // 4 * 4
+    # Four splits make a workgroup, and a compute unit holds two such workgroups. A launch a
+    # little over a whole number of workgroups per compute unit (288 of them: 32 of the 256
+    # units get a second one and finish last) is cut down to that whole number; measured on
+    # an MI355X at 8 kv heads, ms per step of a 4B-sized model: 12 rows behind 2,048 keys 3.29
+    # with 12 splits (288 workgroups) against 3.16 with 8 (192), behind 8,192 keys 5.82 against
+    # 4.97; 6 rows 2.75 with 24 splits (288) against 2.65 with 16 (192), 3.96 against 3.55; 24
+    # rows 4.40 with 8 splits (384) against 4.20 with 4 (192).
+    tasks = waves                                   # (row block, kv head, chunk of heads)
+    groups = tasks * (n // 4)
+    if groups > n_units and groups % n_units and (groups % n_units) * 4 < n_units * 3:
+        fewer = (n_units * (groups // n_units) // tasks) * 4
+        if fewer >= 4:
+            n = fewer
     split_len = ((max_keys + n - 1) // n + 15) // 16 * 16
     return split_len, ((max_keys + split_len - 1) // split_len + 3) // 4 * 4
 
@@ -110,13 +123,14 @@ def plan_key_splits(n_blocks, n_kv_heads, group, max_keys, target_waves=1024, mi
 class NormOwed:
     """Rows that are still owed their RMSNorm factor: ``x`` [M, dim] = bfloat16(h * gain) of the
     rows h of the residual stream, and ``ssq`` [M, tiles rounded up to 4], float32 partial sums
-    of h^2 over tiles of 16 columns (the padding is never read). The factor 1 / sqrt(sum(ssq) / dim + eps) is one number per row, so the
+    of h^2 over ``tiles`` runs of columns (16 each, or fewer where the product that made them gave its workgroups fewer weight rows; the padding is never read). The factor 1 / sqrt(sum(ssq) / dim + eps) is one number per row, so the
     product that consumes the rows applies it to its sums (``HipKernels.linear`` and
     ``linear_swiglu`` take a NormOwed where they take x). Made by ``linear_add_norm``."""
-    __slots__ = ("x", "ssq", "dim", "eps")
+    __slots__ = ("x", "ssq", "dim", "eps", "tiles")
 
-    def __init__(self, x, ssq, dim, eps):
+    def __init__(self, x, ssq, dim, eps, tiles=None):
         self.x, self.ssq, self.dim, self.eps = x, ssq, dim, eps
+        self.tiles = tiles if tiles is not None else (dim + 15) // 16      # partial sums per row
 
     @property
     def shape(self):
@@ -231,6 +245,7 @@ class HipKernels:
         self.split_target_waves, self.split_min_keys = 1024, 64
         self.addnorm_waves = 0          # waves of such a projection, override
         self.addnorm_splits = 0         # workgroups that share one tile's K in it, override
+        self.addnorm_tile_rows = 0      # weight rows of a workgroup in it (8 to 16), override
         # arrival counts of those workgroups, one per tile of 16 outputs: zero between launches
         # (the last to arrive leaves it so). All launches of this kernel set share them, so
         # they must not overlap: one stream, as everywhere in this package.
@@ -422,15 +437,16 @@ class HipKernels:
 
     _SK_SWIGLU, _SK_SCALED = 1, 2
 
-    def _by_tile(self, w):
+    def _by_tile(self, w, h=16):
         """(the tensor a skinny product reads, 1 if it lies by tile else 0) for weight ``w``
-        [N, K] bfloat16. The copy by tile is made at the first call for a weight (not while a
-        graph is being captured: such a call reads the weight row by row); the entry keeps the
-        weight alive, so its address cannot come to mean another tensor."""
+        [N, K] bfloat16, in tiles of ``h`` rows: [N / h, K / 32, h, 32]. The copy by tile is made
+        at the first call for a weight and a tile height (not while a graph is being captured:
+        such a call reads the weight row by row); the entry keeps the weight alive, so its
+        address cannot come to mean another tensor."""
         N, K = w.shape
-        if N % 16 or K % 32 or w.dtype != torch.bfloat16 or not w.is_contiguous():
+        if N % h or K % 32 or w.dtype != torch.bfloat16 or not w.is_contiguous():
             return w, 0
-        key = (w.data_ptr(), N, K)
+        key = (w.data_ptr(), N, K, h)
         entry = self._packed.get(key)
         if entry is not None and entry[2] == w._version:
             return entry[1], 1
@@ -438,7 +454,7 @@ class HipKernels:
         if (not self.pack_weights or N * K < self.pack_min_elements or torch.cuda.is_current_stream_capturing()):
             return w, 0
         try:
-            tiled = w.view(N // 16, 16, K // 32, 32).permute(0, 2, 1, 3).contiguous()
+            tiled = w.view(N // h, h, K // 32, 32).permute(0, 2, 1, 3).contiguous()
         except torch.cuda.OutOfMemoryError:
             # no room for second copies (weights and cache fill the GPU): no new ones from now
             # on; the weights that have one keep using it
@@ -558,7 +574,7 @@ class HipKernels:
             return None, 0, 0, 0.0
         if owed.dim != K:
             raise KernelError(f"rows owed a norm over {owed.dim} elements meet a product over {K}")
-        tiles = (owed.dim + 15) // 16
+        tiles = owed.tiles
         self._want(owed.ssq, "sums of squares", torch.float32, (M, (tiles + 3) // 4 * 4))
         return _ptr(owed.ssq), tiles, owed.dim, owed.eps
 
@@ -585,14 +601,20 @@ class HipKernels:
         self._want(w, "weight", None, (N, K))
         self._want(residual, "residual", torch.float32, (M, N))
         self._want(gain, "norm weight", torch.float32, (N,))
-        tiles = (N + 15) // 16
+        tile_h, k_splits = self._addnorm_shape(N, K, M)
+        if self.addnorm_tile_rows:
+            tile_h = self.addnorm_tile_rows
+        if self.addnorm_splits:
+            k_splits = self.addnorm_splits
+        if (N + tile_h - 1) // tile_h > 4096:
+            tile_h = 16                     # a row's sums of squares are at most 16 segments of 256 tiles
+        tiles = (N + tile_h - 1) // tile_h
         x_out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
         ssq_out = torch.empty((M, (tiles + 3) // 4 * 4), dtype=torch.float32, device=self.device)
         n_waves = self.addnorm_waves or 8
         while n_waves > 1 and K // n_waves < 128:
             n_waves //= 2
         ssq, in_tiles, dim, in_eps = self._owed_args(owed, M, K)
-        k_splits = self.addnorm_splits or self._addnorm_splits(tiles, K, M)
         while k_splits > 1 and K // (k_splits * n_waves) < 128:
             k_splits //= 2
         sums = count = None
@@ -602,17 +624,44 @@ class HipKernels:
                                   "that K can be split for")
             sums = torch.empty((tiles, k_splits, 256), dtype=torch.float32, device=self.device)
             count = self._split_count
-        wt, tiled = self._by_tile(w)
+        wt, tiled = self._by_tile(w, tile_h)
         self.forms[f"add_norm:{k_splits}"] += 1
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(yx), _ptr(wt), None, c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(in_tiles),
             c_int(dim), c_float(in_eps), _ptr(residual), _ptr(gain), _ptr(x_out), _ptr(ssq_out),
-            c_int(k_splits), _ptr(sums), _ptr(count), c_int(tiled | yx_layout), self._stream()),
+            c_int(k_splits), _ptr(sums), _ptr(count), c_int(tiled | yx_layout), c_int(tile_h), self._stream()),
             f"linear_add_norm [{M}x{K}] x [{N}x{K}]^T")
-        return NormOwed(x_out, ssq_out, N, eps)
+        return NormOwed(x_out, ssq_out, N, eps, tiles)
+
+    def _addnorm_shape(self, N, K, M):
+        """(weight rows of a workgroup, workgroups that share a tile's K) of ``linear_add_norm``.
+        A workgroup's 16-row product may hold fewer than 16 weight rows: a narrow output then
+        spreads over more compute units (2,560 outputs are 160 tiles of 16 rows, which leave 96
+        of 256 compute units idle while the others stream at what one compute unit can take, or
+        256 tiles of 10). Heights that divide N (the copy by tile wants whole tiles), from 16
+        down to 8; the cost of a shape is what its busiest compute unit streams, its share of
+        the weights and its reading of x, plus the meeting if K is split. Measured alone inside
+        replayed graphs, weights from memory, us at 8 rows (16 rows per workgroup, its best
+        split of K / 10 rows, K whole): [2,560 x 9,728] 15.4 / 12.8, [2,560 x 4,096] 7.7 / 7.4,
+        [5,120 x 8,192] 20.9 / 20.1, [5,120 x 25,600] 53.6 / 58.1 (there 16 rows in four parts of
+        K stay); 8 rows per workgroup (320 or 640 workgroups) lose everywhere."""
+        best, best_cost = (16, 1), None
+        for h in range(16, 7, -1):
+            if h != 16 and (N % h or M < 5):
+                # (up to 4 rows whole tiles stay ahead inside a step, measured at 4B-sized layers:
+                # 2.34 against 2.37 ms at one row, 2.51 against 2.53 at four; from 6 rows on the
+                # lower tiles win: 2.76 against 2.83 ms at 8 rows, 3.55 against 3.62 at 16)
+                continue
+            tiles = -(-N // h)
+            splits = self._addnorm_splits(tiles, K, M, h)
+            rounds = -(-tiles * splits // 256)
+            cost = rounds * (K / splits) * (h + 0.5 * min(M, 16)) / 16 + (3000 * 8 / max(M, 8) if splits > 1 else 0)
+            if best_cost is None or cost < best_cost * 0.97:
+                best, best_cost = (h, splits), cost
+        return best
 
     @staticmethod
-    def _addnorm_splits(tiles, K, M):
+    def _addnorm_splits(tiles, K, M, h=16):
         """Workgroups that share one tile's K in ``linear_add_norm``: 1, 2 or 4, whichever gives
         the busiest of the GPU's 256 compute units the least to stream, with the meeting in
         memory priced at some 3,000 elements of K (less at more rows, where streaming is
@@ -627,7 +676,7 @@ class HipKernels:
             if splits > 1 and K // (splits * 8) < 256:
                 continue
             rounds = -(-tiles * splits // 256)
-            cost = rounds * K / splits + (3000 * 8 / max(M, 8) if splits > 1 else 0)
+            cost = rounds * (K / splits) * h / 16 + (3000 * 8 / max(M, 8) if splits > 1 else 0)
             if best_cost is None or cost < best_cost:
                 best, best_cost = splits, cost
         return best
@@ -830,7 +879,8 @@ class HipKernels:
         wt, tiled = self._by_tile(w)
         _check(self._gemm.soc_gemm_bf16_skinny_norm(
             _ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K), c_int(n_waves), ssq, c_int(tiles),
-            c_int(dim), c_float(eps), None, None, None, None, c_int(1), None, None, c_int(tiled), self._stream()),
+            c_int(dim), c_float(eps), None, None, None, None, c_int(1), None, None, c_int(tiled), c_int(16),
+            self._stream()),
             f"linear (norm owed) [{M}x{K}] x [{N}x{K}]^T")
         return out
 

@@ -179,9 +179,23 @@ def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
         assert torch.equal(again, r_s)
     hip.addnorm_splits = 0
     assert int(hip._split_count.abs().sum()) == 0
+    # fewer than 16 weight rows per workgroup (a narrow output over more compute units), from
+    # the weights by tile and row by row: the same sums as with 16
+    kept = hip.pack_min_elements
+    hip.addnorm_splits = 1                       # (K whole, as in `first`: the sums are added in the same order)
+    for rows_, pack in ((16, 1), (10, 1), (8, 1 << 40), (13, 1)):
+        hip.addnorm_tile_rows, hip.pack_min_elements = rows_, pack
+        r_h = res.clone()
+        owed_h = hip.linear_add_norm(y, w, r_h, gain, eps)
+        assert owed_h.tiles == -(-d // rows_)
+        torch.testing.assert_close(r_h, r, atol=0, rtol=0)
+        assert torch.equal(owed_h.x, first.x)
+        torch.testing.assert_close(owed_h.ssq[:, :owed_h.tiles].sum(-1), first.ssq[:, :first.tiles].sum(-1), rtol=1e-5, atol=1e-6)
+    hip.addnorm_tile_rows, hip.pack_min_elements, hip.addnorm_splits = 0, kept, 0
     r = res.clone()
     owed = hip.linear_add_norm(y, w, r, gain, eps)
-    tiles = (d + 15) // 16
+    tiles = owed.tiles                           # runs of 8 to 16 columns: the weight rows of a workgroup
+    assert tiles in {-(-d // h) for h in range(8, 17)} and (M >= 5 or tiles == -(-d // 16))
     assert isinstance(owed, NormOwed) and owed.ssq.shape == (M, (tiles + 3) // 4 * 4)
     torch.testing.assert_close(r.double(), want_res, atol=2e-2, rtol=1e-2)
     torch.testing.assert_close(owed.ssq[:, :tiles].double().sum(-1), (r.double() ** 2).sum(-1), atol=1e-6, rtol=1e-5)

@@ -116,3 +116,38 @@ def test_k_is_split_over_workgroups_only_where_it_pays():
     assert [rule(160, 9728, M) for M in (1, 8, 12, 16)] == [1, 1, 4, 4]
     assert {rule(160, 4096, M) for M in (1, 8, 16)} == {1}
     assert rule(320, 25600, 8) == 4 and rule(320, 8192, 8) == 4
+
+
+def test_key_splits_leave_no_ragged_second_round_of_workgroups():
+    """Four splits make a workgroup and a compute unit holds two: a plan a little over a whole
+    number of workgroups per compute unit is cut down to that number (8 kv heads, groups of 4:
+    6 rows would take 24 splits = 288 workgroups and take 20 = 240; 12 rows take 8 = 192, not
+    12 = 288; 24 rows take 4 = 192, not 8 = 384); plans that fill whole rounds stay."""
+    def groups(rows, keys):
+        return rows * 8 * plan_key_splits(rows, 8, 4, keys)[1] // 4
+    for keys in (2048, 8192):
+        assert plan_key_splits(6, 8, 4, keys)[1] == 20 and plan_key_splits(12, 8, 4, keys)[1] == 8
+        assert plan_key_splits(24, 8, 4, keys)[1] == 4 and plan_key_splits(8, 8, 4, keys)[1] == 16
+        for rows in range(1, 65):
+            g = groups(rows, keys)
+            assert g <= 256 or g % 256 == 0 or (g % 256) * 4 >= 256 * 3 or plan_key_splits(rows, 8, 4, keys)[1] == 4, (rows, keys, g)
+
+
+def test_weight_rows_of_a_workgroup_in_the_projections_with_a_residual_epilogue():
+    """2,560 outputs are 160 tiles of 16 rows, which leave 96 of 256 compute units idle, or 256 of
+    10: from 5 rows of x on the lower tile is taken where it divides the width; widths that fill
+    the GPU with tiles of 16 keep them; the long K of a 32B-sized down projection stays in four
+    parts of 16-row tiles."""
+    from socrates_amd.kernels import HipKernels
+
+    class Rules:
+        _addnorm_splits = staticmethod(HipKernels._addnorm_splits)
+    shape = lambda N, K, M: HipKernels._addnorm_shape(Rules, N, K, M)
+    assert shape(2560, 9728, 8) == (10, 1) and shape(2560, 4096, 16) == (10, 1)
+    assert shape(2560, 9728, 1) == (16, 1) and shape(2560, 9728, 4)[0] == 16
+    assert shape(4096, 4096, 8) == (16, 1) and shape(4096, 12288, 16) == (16, 1)
+    assert shape(5120, 8192, 8) == (10, 1) and shape(5120, 25600, 8) == (16, 4)
+    for N in (64, 72, 100, 2560, 5000, 151936):
+        for M in (1, 5, 16):
+            h, s = shape(N, 4096, M)
+            assert 8 <= h <= 16 and (h == 16 or N % h == 0) and s in (1, 2, 4)

@@ -215,11 +215,11 @@ def wider(request, tmp_path_factory):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_layers_of_the_larger_models(wider, dtype, live):
     """Widths 4,096 (K of 4,096 and 12,288) and 5,120 with 64 query heads (K of 5,120 in two
-    halves per wave, 8,192, and 25,600 split over four workgroups per tile): decode steps of
+    halves per wave, 8,192 into 5,120 outputs as 512 workgroups of 10 weight rows, and 25,600): decode steps of
     1, 8 and 40 rows through captured graphs, every logit against the plain implementation."""
     name, folder, cfg, w, prompts, want = wider
     forms = () if dtype == torch.float32 else \
         ("sweep", "sweep_swiglu", "add_norm", "fused_attention") if live <= 16 else ("parts_of_k", "fused_attention")
     ops = decode_rows_through_graphs(folder, cfg, w, prompts, want, dtype, live, forms)
-    if dtype == torch.bfloat16 and name == "32b" and live == 8:
-        assert ops.forms["add_norm:4"] >= 1, dict(ops.forms)     # K = 25,600 in four parts
+    if dtype == torch.bfloat16 and live <= 16:
+        assert any(k.startswith("add_norm") for k in ops.forms), dict(ops.forms)
