@@ -557,13 +557,13 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     }
 
     // Where four outputs of a row go: element `at` = (token * Hq + head) * D + d of out
-    // [N, Hq * D], or (out_tiled: at most 16 tokens) the same element of out [Hq * D / 32, 16, 32],
+    // [N, Hq * D], or (out_tiled = R > 0: at most R tokens) the same element of out [Hq * D / 32, R, 32],
     // the layout in which the product that follows reads 64 bytes of every row side by side.
     auto out_at = [&](size_t at) -> bf16* {
         if (!out_tiled) return out + at;
         const size_t width = (size_t)Hq * D, tok = at / width;
         const int col = (int)(at - tok * width);
-        return out + ((size_t)(col / 32) * 16 + tok) * 32 + col % 32;
+        return out + ((size_t)(col / 32) * out_tiled + tok) * 32 + col % 32;
     };
     f32x4_t o[RT][DV];
     float m[RT], l[RT];
@@ -952,8 +952,8 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 // tokens per block (the blocks may cover some of the N tokens only; the others' outputs are
 // not touched), and `arrivals`, one int per task (row block x kv head x chunk of 16 heads),
 // zero before the call and zero again after it; calls that may run at the same time need
-// arrival counts of their own. out_tiled (N <= 16, Hq * D a multiple of 32): out is written
-// [Hq * D / 32, 16, 32] instead of [N, Hq * D], for a product that reads its x by tile.
+// arrival counts of their own. out_tiled = R (0: no; N <= R <= 64, Hq * D a multiple of 32): out is
+// written [Hq * D / 32, R, 32] instead of [N, Hq * D], for a product that reads its x by tile.
 SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const void* v_pool,
                                         const int* block_table, int table_width, const int* token_rows,
                                         const int* positions, const int* row_blocks, int n_row_blocks,
@@ -962,7 +962,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
                                         int n_splits, int row_tiles, int group_pad_log2, int out_tiled,
                                         hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
-    if (out_tiled && (N > 16 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
+    if (out_tiled && (out_tiled < 0 || N > out_tiled || out_tiled > 64 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
         return (int)hipErrorInvalidValue;
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
@@ -1027,7 +1027,7 @@ SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, 
         return (int)hipErrorNotSupported;
     } else {
         if (N <= 0) return 0;
-        if (out_tiled && (N > 16 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
+        if (out_tiled && (out_tiled < 0 || N > out_tiled || out_tiled > 64 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
         if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || (split_len != 0 && split_len < 16) || split_len % 16)
             return (int)hipErrorInvalidValue;
         if (n_splits > 1 && n_splits % 4) return (int)hipErrorInvalidValue;

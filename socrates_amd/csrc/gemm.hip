@@ -946,7 +946,8 @@ __global__ void __launch_bounds__(1024)
 gemm_bf16_sweep_parts_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, float* __restrict__ P,
                              int M, int N, int K, SwParts pl, int layout) {
     extern __shared__ __attribute__((aligned(16))) float parts_red[];          // [tile parity][MT][wave][lane][4]
-    const bool w_tiled = layout & SK_W_TILED;
+    const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED;
+    const int x_rows = layout >> 8;                     // x by tile: [K / 32][x_rows][32], x_rows >= M a multiple of 16
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int n_waves = blockDim.x / SOC_WAVE;
     const int part = blockIdx.x % pl.parts, g = blockIdx.x / pl.parts, G = gridDim.x / pl.parts;
@@ -955,21 +956,25 @@ gemm_bf16_sweep_parts_kernel(const bf16* __restrict__ X, const bf16* __restrict_
     const int k_begin = part * pl.k_part + wave * pl.k_per_wave, k_end = min(part_end, k_begin + pl.k_per_wave);
     const int n_sub = pl.tiles > g ? (pl.tiles - g + G - 1) / G : 0;
     const __amdgpu_buffer_rsrc_t x_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, M * K * 2, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(X), (short)0, (x_tiled ? x_rows : M) * K * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16*>(W), (short)0, (int)((size_t)N * K * 2), 0x00020000);
     const int w_rs = w_tiled ? 32 : K, w_ss = w_tiled ? 512 : 32;
+    const int x_rs = x_tiled ? 32 : K, x_ss = x_tiled ? 32 * x_rows : 32;
     uint4 xr[MT][MAXS];
     uint32_t k_off[MAXS];
 #pragma unroll
     for (int s = 0; s < MAXS; ++s) {
         const int k = k_begin + 32 * s + lk;
         k_off[s] = k < k_end ? (uint32_t)((((k_begin / 32 + s) * w_ss) + li * w_rs + lk) * 2) : SW_NOWHERE;
-        // (a row beyond M lies beyond the descriptor's end)
+        // (row by row, a row beyond M lies beyond the descriptor's end; by tile, a row from M on
+        // holds anything or lies beyond x_rows, and its sums are never stored)
 #pragma unroll
         for (int t = 0; t < MT; ++t)
             xr[t][s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                           x_rsrc, k < k_end ? (uint32_t)(((t * 16 + li) * K + k) * 2) : SW_NOWHERE, 0, 0));
+                           x_rsrc, k < k_end && (!x_tiled || t * 16 + li < x_rows)
+                               ? (uint32_t)(((k / 32) * x_ss + (t * 16 + li) * x_rs + k % 32) * 2)
+                               : SW_NOWHERE, 0, 0));
     }
     auto load_w = [&](uint4 (&wb)[MAXS], int q) {
         const bool live = q < n_sub;
@@ -1043,11 +1048,14 @@ SOC_EXPORT int soc_gemm_sweep_parts_plan(int M, int N, int K, int* parts, int* k
 }
 
 // P [parts, M, N] float32 = the partial sums of X [M <= 64, K] times W [N, K] transposed, part p
-// over the p-th run of ceil(K / 32 / parts) * 32 elements of K. layout: SK_W_TILED or 0.
+// over the p-th run of ceil(K / 32 / parts) * 32 elements of K. layout: SK_W_TILED; SK_X_TILED with
+// R << 8: x lies [K / 32][R][32], R a multiple of 16 from M to 64 (K a multiple of 32).
 SOC_EXPORT int soc_gemm_bf16_sweep_parts(const void* X, const void* W, float* P, int M, int N, int K, int parts,
                                          int k_per_wave, int groups, int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if ((layout & ~SK_W_TILED) || ((layout & SK_W_TILED) && (N % 16 || K % 32))) return (int)hipErrorInvalidValue;
+    const int x_rows = layout >> 8;
+    if (((layout & 0xff) & ~(SK_W_TILED | SK_X_TILED)) || ((layout & SK_W_TILED) && (N % 16 || K % 32))) return (int)hipErrorInvalidValue;
+    if ((layout & SK_X_TILED) ? (K % 32 || x_rows < M || x_rows > 64 || x_rows % 16) : x_rows != 0) return (int)hipErrorInvalidValue;
     if (M > 64 || K % 8 || K < 8 || !P) return (int)hipErrorInvalidValue;
     if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;
     if (parts < 1 || groups < 1 || parts * groups > 65535 || k_per_wave < 32 || k_per_wave % 32)
@@ -1113,7 +1121,7 @@ gemm_bf16_stream_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
     constexpr bool SWIGLU = MODE & SK_SWIGLU;
     constexpr int SUB = SWIGLU ? 2 : 1, J = T / SUB, NW = 8;
     static_assert(T % SUB == 0, "whole pairs");
-    const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED;
+    const bool w_tiled = layout & SK_W_TILED, x_tiled = layout & SK_X_TILED, c_tiled = layout & SK_C_TILED;
     __shared__ __attribute__((aligned(16))) float red[2][NW][MT][256];   // [tile parity][wave][row block][lane][4]
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / SOC_WAVE), lane = tid % SOC_WAVE;
     const int g = blockIdx.x, G = gridDim.x;
@@ -1207,8 +1215,10 @@ gemm_bf16_stream_kernel(const bf16* __restrict__ X, const bf16* __restrict__ W, 
                     if (m < M && col < half) {
                         const float a0 = s0 * (held[0] / (1.0f + expf(-held[0])));
                         const float a1 = s1 * (held[1] / (1.0f + expf(-held[1])));
-                        C[(size_t)m * half + col] = from_float<TC>(a0);
-                        if (col + 1 < half) C[(size_t)m * half + col + 1] = from_float<TC>(a1);
+                        // (by tile: [half / 32][16 MT][32], for the product that reads it next)
+                        TC* at = c_tiled ? C + ((size_t)(col / 32) * (16 * MT) + m) * 32 + col % 32 : C + (size_t)m * half + col;
+                        at[0] = from_float<TC>(a0);
+                        if (col + 1 < half) at[1] = from_float<TC>(a1);
                     }
                 } else {
                     const int n = tile_no[t] * 16 + c2;
@@ -1238,12 +1248,13 @@ SOC_EXPORT int soc_gemm_stream_plan(int M, int N, int K, int swiglu, int* workgr
 // C = X [M <= 64, K] times W [N, K] transposed, in c_dtype (0 float32, 1 bfloat16), or with
 // mode SK_SWIGLU C [M, N / 2] = silu(gate) * up over weight rows that alternate in blocks of 16
 // (bfloat16 out). layout: SK_W_TILED, and SK_X_TILED: x is laid out [K / 32][R][32] with R = 32 for
-// M <= 32, 48 for M <= 48 and 64 above (K a multiple of 32). The matrices lie below 4 GiB.
+// M <= 32, 48 for M <= 48 and 64 above (K a multiple of 32); SK_C_TILED (with SK_SWIGLU, N a multiple of
+// 64): C is written [N / 64][R][32] with the same R. The matrices lie below 4 GiB.
 SOC_EXPORT int soc_gemm_bf16_stream(const void* X, const void* W, void* C, int M, int N, int K, int c_dtype,
                                     int mode, int workgroups, int per_wg, int layout, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if ((layout & ~(SK_W_TILED | SK_X_TILED)) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) ||
-        ((layout & SK_X_TILED) && K % 32))
+    if ((layout & ~(SK_W_TILED | SK_X_TILED | SK_C_TILED)) || ((layout & SK_W_TILED) && (N % 16 || K % 32)) ||
+        ((layout & SK_X_TILED) && K % 32) || ((layout & SK_C_TILED) && (!(mode & SK_SWIGLU) || N % 64)))
         return (int)hipErrorInvalidValue;
     if (M > 64 || K % 8 || K < 8 || !C) return (int)hipErrorInvalidValue;
     if (((size_t)N + 32) * K * 2 >= 0xfffffff0ull || (size_t)64 * K * 2 >= 0xfffffff0ull) return (int)hipErrorInvalidValue;

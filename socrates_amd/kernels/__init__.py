@@ -389,8 +389,9 @@ class HipKernels:
                         lambda: self._k_outermost(plan, xt, w_gate_up, torch.empty((M, N // 2), dtype=self.dtype, device=self.device), True),
                         lambda: self.swiglu(torch.mm(xr, w_gate_up.t()), interleave))
                 if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan, True)):
-                    out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
-                    return self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
+                    out = self._swiglu_out(M, N, by_tile)
+                    self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
+                    return out
             x = x.by_rows()
         M, K = x.shape
         N = w_gate_up.shape[0]
@@ -431,11 +432,20 @@ class HipKernels:
                         lambda: self._k_outermost(plan, x, w_gate_up, torch.empty((M, N // 2), dtype=self.dtype, device=self.device), True),
                         lambda: self.swiglu(torch.mm(x, w_gate_up.t()), interleave))
                 if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan, True, by_tile=False)):
-                    out = torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
-                    return self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
+                    out = self._swiglu_out(M, N, by_tile)
+                    self._k_outermost(plan, x, w_gate_up, out, True, what="linear_swiglu")
+                    return out
         return self.swiglu(self.linear(owed if owed is not None else x, w_gate_up), interleave)
 
     _SK_SWIGLU, _SK_SCALED = 1, 2
+
+    def _swiglu_out(self, M, N, by_tile):
+        """Where the activation of 17 to 64 rows goes: [M, N / 2], or by tile where the caller
+        hands it to one projection and nowhere else."""
+        if by_tile and self.rows_by_tile and N % 64 == 0:
+            rows = (M + 15) // 16 * 16
+            return RowsByTile(torch.empty((N // 64, rows, 32), dtype=self.dtype, device=self.device), M, N // 2)
+        return torch.empty((M, N // 2), dtype=self.dtype, device=self.device)
 
     def _by_tile(self, w, h=16):
         """(the tensor a skinny product reads, 1 if it lies by tile else 0) for weight ``w``
@@ -535,6 +545,8 @@ class HipKernels:
     def _k_outermost(self, plan, x, w, out, swiglu=False, what="linear"):
         (M, K), N = x.shape, w.shape[0]
         wt, tiled = self._by_tile(w)
+        if isinstance(out, RowsByTile):                  # the activation by tile, for the projection behind it
+            out, tiled = out.data, tiled | 4
         if isinstance(x, RowsByTile):
             self._want(x.data, "x by tile", torch.bfloat16, (K // 32, (M + 15) // 16 * 16, 32))
             x, tiled = x.data, tiled | 2
@@ -561,6 +573,10 @@ class HipKernels:
         parts, kpw, groups = plan
         out = torch.empty((parts, M, N), dtype=torch.float32, device=self.device)
         wt, tiled = self._by_tile(w)
+        if isinstance(x, RowsByTile):
+            rows = x.data.shape[1]
+            self._want(x.data, "x by tile", torch.bfloat16, (K // 32, rows, 32))
+            x, tiled = x.data, tiled | 2 | (rows << 8)
         self.forms[f"parts_of_k:{parts}"] += 1
         _check(self._gemm.soc_gemm_bf16_sweep_parts(_ptr(x), _ptr(wt), _ptr(out), c_int(M), c_int(N), c_int(K),
                                                     c_int(parts), c_int(kpw), c_int(groups), c_int(tiled),
@@ -757,6 +773,15 @@ class HipKernels:
                             lambda: torch.mm(xr, w.t()) if odt == torch.bfloat16 else torch.mm(xr, w.t(), out_dtype=odt))
                     if choice != "library" and (choice == "own" or self._stream_default(M, N, K, plan)):
                         return self._k_outermost(plan, x, w, torch.empty((M, N), dtype=odt, device=self.device))
+            if (x.data.shape[1] > 16 and w.dim() == 2 and w.dtype == torch.bfloat16 and x.shape[1] == w.shape[1]
+                    and allow_partial and self.library_gemm and not (row_tiles or n_waves or k_splits or self._tuning)):
+                # 17 to 64 rows by tile (from the decode attention or the gate / up product) into a
+                # projection that ends a branch: the sweep over parts of K reads them so
+                (M, K), N = x.shape, w.shape[0]
+                plan = self._parts_plan(M, N, K)
+                if plan is not None and self.product_choice.get((M, N, K, out_dtype or self.dtype, True)) != "library":
+                    self._want(w, "weight")
+                    return self._sweep_parts(plan, x, w)
             x = x.by_rows()
         self._want(x, "x")
         self._want(w, "weight")
@@ -1128,8 +1153,9 @@ class HipKernels:
                 return None
             part_o = torch.empty((N, Hq, n_splits // 4, D), dtype=torch.float32, device=self.device)
             part_ml = torch.empty((N, Hq, n_splits // 4, 2), dtype=torch.float32, device=self.device)
-        tiled = bool(by_tile and self.rows_by_tile and N <= 16 and (Hq * D) % 32 == 0)
-        out = torch.empty((Hq * D // 32, 16, 32) if tiled else (N, Hq * D), dtype=self.dtype, device=self.device)
+        tile_rows = (N + 15) // 16 * 16 if by_tile and self.rows_by_tile and N <= 64 and (Hq * D) % 32 == 0 else 0
+        tiled = tile_rows > 0
+        out = torch.empty((Hq * D // 32, tile_rows, 32) if tiled else (N, Hq * D), dtype=self.dtype, device=self.device)
         self.last_attention_kernel = ("fused", 1)
         self.forms[f"fused_attention:{n_splits}"] += 1
         _check(lib.soc_paged_attention_decode_fused(
@@ -1138,7 +1164,7 @@ class HipKernels:
             _ptr(part_ml), _ptr(self._split_count), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
             c_float(scale), c_int(int(window) if window else 0), c_int(split_len), c_int(n_splits), c_int(gpl),
             _ptr(q_gain), _ptr(k_gain), _ptr(rope_table), c_float(eps), c_int(1 if write else 0),
-            c_int(1 if tiled else 0), self._stream()), "decode_attention")
+            c_int(tile_rows), self._stream()), "decode_attention")
         return RowsByTile(out, N, Hq * D) if tiled else out
 
     def paged_attention(self, q, slot, ctx, scale, window=None, terms=None):

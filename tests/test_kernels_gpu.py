@@ -362,6 +362,20 @@ def test_normed_rows_by_tile_into_the_products_with_k_outermost(kernel_sets, M, 
         assert torch.equal(hip.linear(tiled, w, out_dtype=torch.float32), hip.linear(rows, w, out_dtype=torch.float32))
         assert torch.equal(hip.linear_swiglu(tiled, w, 16), hip.linear_swiglu(rows, w, 16))
         assert hip.forms["stream"] == 4 and hip.forms["stream_swiglu"] == 2, dict(hip.forms)
+        # the activation of the gate / up product by tile is the same values, and a projection that
+        # ends a branch reads rows by tile in its sweep over parts of K: the same bits
+        act_t, act_r = hip.linear_swiglu(tiled, w, 16, by_tile=True), hip.linear_swiglu(rows, w, 16)
+        if N % 64 == 0:
+            assert isinstance(act_t, RowsByTile) and torch.equal(act_t.by_rows(), act_r)
+        kept_k = hip.parts_min_k
+        hip.parts_min_k = 32
+        try:
+            if hip._parts_plan(M, N, d) is not None:
+                hip.forms.clear()
+                assert torch.equal(hip.linear(tiled, w, allow_partial=True), hip.linear(rows, w, allow_partial=True))
+                assert sum(v for k, v in hip.forms.items() if k.startswith("parts_of_k")) == 2, dict(hip.forms)
+        finally:
+            hip.parts_min_k = kept_k
         # a consumer that wants partial sums, or the library, gets the rows
         parts = hip.linear(tiled, w, allow_partial=True)
         close(parts.sum(0) if parts.dim() == 3 else parts, rows.float() @ w.float().T, torch.bfloat16)
@@ -632,6 +646,7 @@ def test_decode_attention_from_raw_qkv(kernel_sets, Hq, Hkv, D, bs, norm, rope):
                                          slot_a, ctx, 0.2, window, False, by_tile=True)
             if (Hq * D) % 32 == 0:
                 assert type(tiled).__name__ == "RowsByTile" and tiled.shape == (N, Hq * D)
+                assert tiled.data.shape[1] == (N + 15) // 16 * 16
                 assert torch.equal(tiled.by_rows(), got_r)
             else:
                 assert torch.equal(tiled, got_r)
