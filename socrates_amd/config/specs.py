@@ -24,17 +24,22 @@ class RMSNormSpec:
 class RopeSpec:
     """Rotate-half rotary encoding over the first ``rotary_dim`` of each head.
 
-    inv_freq[j] = theta ** (-2j / rotary_dim), pairs are (j, j + rotary_dim/2).
+    inv_freq[j] = theta ** (-2j / rotary_dim) / factor, pairs are (j, j + rotary_dim/2).
+    ``factor`` (1: none; the reference's model has none) stretches the positions a checkpoint was
+    trained on by that much (linear position interpolation).
     """
     head_dim: int
     theta: float
     rotary_dim: int = 0          # 0 means the whole head
+    factor: float = 1.0
 
     def __post_init__(self):
         if self.rotary_dim == 0:
             object.__setattr__(self, "rotary_dim", self.head_dim)
         if self.rotary_dim % 2 or self.rotary_dim > self.head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and <= head_dim {self.head_dim}")
+        if not self.factor > 0:
+            raise ValueError("factor must be positive")
 
 
 @dataclass(frozen=True)

@@ -7,7 +7,8 @@ once to the compute dtype.
 
 The constants of a rotation (inv_freq, and the table of cosines and sines by position
 that the fused decode kernel looks up) belong to (kernel set, theta, rotary_dim), not to
-a layer: all layers with the same rotation share one ``PositionTable``. The reference
+a layer: all layers with the same rotation (theta, rotary size, stretch factor) share one
+``PositionTable``. The reference
 keeps what its captured steps read in module buffers at fixed addresses
 (model/qwen/qwen_kv_cont.py:97-127); here the table is sized once, for the cache's
 longest row, before any step runs (``reserve``), and a kernel set is told when it
@@ -30,10 +31,12 @@ class PositionTable:
     """inv_freq [rotary_dim / 2] and, once reserved, cosines and sines of positions
     0 .. n - 1, float32 [n, 2, rotary_dim / 2], made by the kernel set's own arithmetic."""
 
-    def __init__(self, theta, rotary_dim, ops):
+    def __init__(self, theta, rotary_dim, ops, factor=1.0):
         self.ops = ops
         # The reference's own expression (qwen_kv_cont.py:60), evaluated in float32.
         inv_freq = 1.0 / (theta ** (torch.arange(0, rotary_dim, 2).float() / rotary_dim))
+        if factor != 1.0:
+            inv_freq = inv_freq / factor
         self.inv_freq = inv_freq.to(ops.device)
         self.rows = None
 
@@ -55,11 +58,11 @@ class PositionTable:
         return rows
 
 
-def shared_table(ops, theta, rotary_dim) -> PositionTable:
+def shared_table(ops, theta, rotary_dim, factor=1.0) -> PositionTable:
     per_ops = _SHARED.setdefault(ops, {})
-    key = (float(theta), int(rotary_dim))
+    key = (float(theta), int(rotary_dim), float(factor))
     if key not in per_ops:
-        per_ops[key] = PositionTable(theta, rotary_dim, ops)
+        per_ops[key] = PositionTable(theta, rotary_dim, ops, factor)
     return per_ops[key]
 
 
@@ -70,7 +73,7 @@ class Rope:
 
     def __init__(self, spec: RopeSpec, tensors, ops):
         self.spec, self.ops = spec, ops
-        self.shared = shared_table(ops, spec.theta, spec.rotary_dim)
+        self.shared = shared_table(ops, spec.theta, spec.rotary_dim, spec.factor)
         self.inv_freq = self.shared.inv_freq
         # kernels look cosines and sines up only for a rotation over the whole head
         self._tabled = hasattr(ops, "rope_table") and spec.rotary_dim == spec.head_dim

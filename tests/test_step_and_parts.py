@@ -659,3 +659,39 @@ def test_a_model_with_further_score_terms_and_scaled_embedding_and_logits(kind, 
         full = plain_attention_with_terms(q0, k0, v0, 0.25, slopes=slopes, softcap=5.0,
                                           sinks=weights["model.layers.0.self_attn.sinks"].float().cpu())
         assert (plain_attention_with_terms(q0, k0, v0, 0.25, **terms) - full).abs().max() > 1e-2, drop
+
+
+@pytest.mark.parametrize("kind,dtype", KINDS)
+def test_a_rotation_with_stretched_positions_and_half_a_head(kind, dtype):
+    """RopeSpec(factor=4): positions are divided by 4 (inv_freq / 4), as a rotation by position / 4
+    written out here gives; RopeSpec(rotary_dim=D / 2): the first half of the head is rotated and
+    the rest passes through. Both through the decode path too (the kernel set falls back to the
+    kernels one after the other where its one-kernel form does not apply)."""
+    ops = kernels(kind, dtype)
+    D, T = 64, 23
+    q, k = torch.randn(T, 4, D), torch.randn(T, 2, D)
+    positions = torch.arange(5, 5 + T)
+    dev = lambda t: t.to(dtype).to(ops.device).clone()
+    for spec, rot, factor in ((RopeSpec(D, 1e4, factor=4.0), D, 4.0), (RopeSpec(D, 1e4, rotary_dim=D // 2), D // 2, 1.0)):
+        rope = build_part(spec, {}, ops)
+        qd, kd = dev(q), dev(k)
+        rope.apply(qd, kd, positions.to(torch.int32).to(ops.device))
+        inv_freq = 1.0 / (1e4 ** (torch.arange(0, rot, 2).float() / rot)) / factor
+        ang = positions.float()[:, None] * inv_freq
+        cos, sin = torch.cat([ang.cos()] * 2, -1)[:, None], torch.cat([ang.sin()] * 2, -1)[:, None]
+        for got, x in ((qd, q), (kd, k)):
+            x = x.to(dtype).float()
+            head = x[..., :rot]
+            want = torch.cat([head * cos + torch.cat([-head[..., rot // 2:], head[..., :rot // 2]], -1) * sin, x[..., rot:]], -1)
+            torch.testing.assert_close(got.float().cpu(), want, **TOL[dtype])
+    # inside a model: whole prompt against cut prompt with decoded tokens
+    hidden = 64
+    blocks = []
+    for i, pos in enumerate((RopeSpec(D, 1e4, factor=4.0), RopeSpec(D, 1e4, rotary_dim=D // 2))):
+        att = AttentionSpec(hidden, 2, 1, D, D ** -0.5, RMSNormSpec(D, 1e-6), pos)
+        blocks.append(BlockSpec(att, SwiGLUSpec(hidden, 96), RMSNormSpec(hidden, 1e-6), RMSNormSpec(hidden, 1e-6),
+                                prefix=f"model.layers.{i}."))
+    plan = plan_with(blocks, [RunStep(0, 0), RunStep(1, 1)], hidden)
+    tokens = random_prompts([30], 50, seed=9)[0]
+    _, (whole_run, cut_run) = run_whole_and_cut(plan, ops, tokens, [[30], [11, 1, 1, 16, 1]])
+    torch.testing.assert_close(cut_run, whole_run, **(TOL[dtype] if dtype == torch.float32 else dict(atol=0.1, rtol=5e-2)))
