@@ -604,8 +604,9 @@ class HipKernels:
         yx = owed.x if owed is not None else (tiled_y.data if tiled_y is not None else y)
         (M, K), N = (tiled_y.shape if tiled_y is not None else yx.shape), w.shape[0]
         if not (self.dtype == torch.bfloat16 and yx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N <= 65536 and self.fuse_norms):
-            # (65,536: the sums of squares of a row are summed by one wave per 256 tiles of 16)
+                and 0 < M <= 16 and K % 8 == 0 and K >= 8 and N % 8 == 0 and N <= 65536 and self.fuse_norms):
+            # (65,536: the sums of squares of a row are summed by one wave per 256 tiles of 16;
+            # N % 8: the product that takes the owed rows has N as its K, and reads 8 at a time)
             # (the rows go to one product and nowhere else, as a NormOwed would: they may lie by tile)
             return self.add_rmsnorm(residual, self.linear(y, w, allow_partial=True), gain, eps, by_tile=True)
         if tiled_y is not None:

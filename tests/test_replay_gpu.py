@@ -122,6 +122,25 @@ def test_first_tokens_and_long_decode(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("hidden,inter", [(50, 300), (44, 24)])
+def test_widths_that_are_no_multiple_of_eight(tmp_path, hidden, inter, dtype):
+    """A width of 50 or 44: the bfloat16 products that read eight elements at a time do not
+    apply, and a short step must not leave rows owed their norm to a product that cannot take
+    them (it once did, and the step stopped with an error). Portions, then tokens one by one."""
+    tiny = dict(cfg=dict(architectures=["Qwen3ForCausalLM"], vocab_size=211, hidden_size=hidden,
+                         num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+                         intermediate_size=inter, rms_norm_eps=1e-6, rope_theta=1e4, tie_word_embeddings=True),
+                block_size=8, gain_std=0.1)
+    folder = write_tiny(tmp_path / "m", tiny, seed=hidden)
+    cfg, w = plain.read_folder(folder)
+    prompts = random_prompts([40, 7, 70], cfg["vocab_size"], seed=2)
+    want = {f"r{i}": plain.forward(cfg, w, p) for i, p in enumerate(prompts)}
+    for steps in (trace_portions(prompts, seed=3), trace_tail_decode(prompts, 32)):
+        runner = runner_for(folder, tiny, dtype, 40)
+        compare(replay(runner, steps), want, dtype, f"hidden {hidden}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_captured_decode_steps_follow_the_data(folders, oracle, dtype):
     """Decode-only steps replayed from HIP graphs: every replay is compared with the plain
     oracle, with eager work (prompt portions, other widths, synchronisations) between the
