@@ -290,8 +290,11 @@ def main(argv=None):
     sized = {"qwen3-4b": "Qwen3-4B-sized", "qwen3-8b": "Qwen3-8B-sized", "qwen3-32b": "Qwen3-32B-sized"}.get(
         args.preset, args.preset)
     biggest = max(args.batch, 1 if args.no_points else 64)
+    if args.prefill_tokens + 1 > args.max_len:
+        ap.error(f"--prefill-tokens {args.prefill_tokens} needs --max-len of at least {args.prefill_tokens + 1}")
+    # the timed prefill is one step: the scheduler's portion holds the whole prompt
     config, engine = build_engine(cfg, dtype, biggest, args.max_len, seed=0, compile_=not args.no_graphs,
-                                  block_size=args.block_size)
+                                  chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
     V = config.vocab_size
     engine.runner.ops.fuse_norms = not args.no_fused_norms
     for item_ in args.set:
