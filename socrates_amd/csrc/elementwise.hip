@@ -310,6 +310,29 @@ SOC_EXPORT int soc_scale_softcap(float* x, long long n, float scale, float cap, 
     return soc_last_error();
 }
 
+// Rows that are owed their norm's factor, settled: out[m][c] = x[m][c] / sqrt(sum_t ssq[m][t] /
+// dim + eps), bfloat16 in and out, for a product that cannot apply the factor to its sums (a
+// weight kept in float32, a float32 result). One workgroup per row; every thread adds the row's
+// partial sums in the same order.
+__global__ void settle_owed_kernel(const bf16* __restrict__ x, const float* __restrict__ ssq, int tiles,
+                                   int ssq_stride, bf16* __restrict__ out, int dim, float eps) {
+    const int m = blockIdx.x;
+    float sum = 0.f;
+    for (int t = 0; t < tiles; ++t) sum += ssq[(size_t)m * ssq_stride + t];
+    const float factor = rsqrtf(sum / (float)dim + eps);
+    for (int c = threadIdx.x; c < dim; c += blockDim.x)
+        out[(size_t)m * dim + c] = from_float<bf16>(to_float(x[(size_t)m * dim + c]) * factor);
+}
+
+SOC_EXPORT int soc_settle_owed(const void* x, const float* ssq, int tiles, int ssq_stride, void* out, int M,
+                               int dim, float eps, hipStream_t stream) {
+    if (M <= 0 || dim <= 0) return 0;
+    if (tiles < 1 || ssq_stride < tiles) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(settle_owed_kernel, dim3((unsigned)M), dim3(256), 0, stream, (const bf16*)x, ssq, tiles,
+                       ssq_stride, (bf16*)out, dim, eps);
+    return soc_last_error();
+}
+
 SOC_EXPORT int soc_swiglu(const void* gate_up, void* out, int N, int ff, int interleave, int dtype,
                           hipStream_t stream) {
     const size_t total = (size_t)N * ff;

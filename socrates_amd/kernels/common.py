@@ -30,6 +30,7 @@ _EW_SIGNATURES = {
     "soc_rmsnorm": [P, P, P, I, I, F, I, P],
     "soc_swiglu": [P, P, I, I, I, I, P],
     "soc_scale_softcap": [P, c_longlong, F, F, P],
+    "soc_settle_owed": [P, P, I, I, P, I, I, F, P],
     "soc_qk_norm_rope": [P] * 7 + [I] + [P] * 5 + [I] * 6 + [F, I, P],
     "soc_rope": [P, P, P, I, I, I, I, I, P],
     "soc_kv_write": [P] * 5 + [I, P, P, I, I, I, I, I, P],

@@ -543,17 +543,31 @@ class Products:
         _check(err, f"linear [{M}x{K}] x [{N}x{K}]^T")
         return out
 
+    def settle(self, owed):
+        """The normed rows themselves, bfloat16 [M, dim], of rows still owed their norm's factor."""
+        x = owed.x
+        M, dim = x.shape
+        self._want(x, "x", torch.bfloat16)
+        self._want(owed.ssq, "sums of squares", torch.float32)
+        out = torch.empty_like(x)
+        _check(self._ew.soc_settle_owed(_ptr(x), _ptr(owed.ssq), c_int(owed.tiles), c_int(owed.ssq.shape[1]), _ptr(out),
+                                        c_int(M), c_int(dim), c_float(owed.eps), self._stream()), "settle")
+        return out
+
     def _linear_owed(self, owed, w, out_dtype, n_waves=0):
         """x' [M <= 16, K] of a NormOwed times w [N, K] transposed, the norm's factor applied
-        to the sums: one skinny product, bfloat16 out."""
+        to the sums: one skinny product, bfloat16 out. Where that product does not apply (a
+        float32 weight or result) the rows are settled and go the ordinary way."""
         x = owed.x
         self._want(x, "x", torch.bfloat16)
-        self._want(w, "weight", torch.bfloat16)
         if w.dim() != 2 or x.shape[1] != w.shape[1]:
             raise KernelError(f"linear: x {tuple(x.shape)} does not fit weight {tuple(w.shape)}")
         (M, K), N = x.shape, w.shape[0]
-        if out_dtype != torch.bfloat16 or not 0 < M <= 16 or K % 8:
-            raise KernelError("rows owed a norm go to bfloat16 products of at most 16 rows")
+        if w.dtype != torch.bfloat16 or out_dtype != torch.bfloat16 or not 0 < M <= 16 or K % 8:
+            # (a weight kept in float32 because the file stores it so, a float32 result: the
+            # product that takes those cannot apply the factor to its sums; the rows are settled first)
+            return self.linear(self.settle(owed), w, out_dtype)
+        self._want(w, "weight", torch.bfloat16)
         out = torch.empty((M, N), dtype=torch.bfloat16, device=self.device)
         plan = self._sweep_plan(M, N, K) if not n_waves else None
         if plan is not None:

@@ -231,6 +231,20 @@ def test_linear_add_norm_and_products_of_owed_rows(kernel_sets, M, d, K, eps):
         owed3 = hip.linear_add_norm(owed, w3, r3, gain3, 1e-5)
         torch.testing.assert_close(r3.double(), res3.double() + normed @ w3.double().T, atol=2e-2, rtol=2e-2)
         torch.testing.assert_close(owed3.x, (r3 * gain3).to(torch.bfloat16), atol=0, rtol=0)
+        # a consumer that cannot apply the factor to its sums (a weight kept in float32 because
+        # its file stores it so, a float32 result) gets the rows settled (it once stopped with an error)
+        close(hip.settle(owed), normed, torch.bfloat16)
+        close(hip.linear(owed, w2.float()), normed @ w2.double().T, torch.bfloat16)
+        close(hip.linear(owed, w2, out_dtype=torch.float32), normed @ w2.double().T, torch.bfloat16)
+        # (three roundings to bfloat16 on this way: the settled rows, the gate and up sums before
+        # the activation kernel, the result; bounded against each row's largest value at three
+        # times what the products with one rounding are held to, 6e-3)
+        act = hip.linear_swiglu(owed, wgu.float(), 16)
+        assert ((act.double() - want).abs() / want.abs().amax(-1, keepdim=True)).max() < 1.8e-2
+        r4 = res3.clone()
+        rows4 = hip.linear_add_norm(owed, w3.float(), r4, gain3, 1e-5)
+        torch.testing.assert_close(r4.double(), res3.double() + normed @ w3.double().T, atol=2e-2, rtol=2e-2)
+        assert not isinstance(rows4, NormOwed)
     # more than 16 rows, or the switch off: the same call is product, then sum and norm
     hip.fuse_norms = False
     r = res.clone()

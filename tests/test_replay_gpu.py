@@ -140,6 +140,34 @@ def test_widths_that_are_no_multiple_of_eight(tmp_path, hidden, inter, dtype):
         compare(replay(runner, steps), want, dtype, f"hidden {hidden}")
 
 
+@pytest.mark.parametrize("which", ["all", "some", "head"])
+def test_matrices_stored_in_32_bit_under_a_bfloat16_run(tmp_path, which):
+    """A file that holds all, some, or the first and last of its matrices in 32-bit floats: they
+    stay so, and a bfloat16 run multiplies with them through the float32 product. Short steps
+    must not hand such a product rows that are owed their norm (they once did, and the step
+    stopped with an error). Mixed steps, then tokens one by one, against the plain run."""
+    import random
+    import warnings
+    from safetensors.torch import load_file, save_file
+    tiny = TINIES["B"]
+    folder = write_tiny(tmp_path / "m", tiny, seed=9)
+    tensors = load_file(str(folder / "model.safetensors"))
+    rng = random.Random(3)
+    for k in list(tensors):
+        if tensors[k].dim() == 2 and (which == "all" or (which == "some" and rng.random() < 0.4) or
+                                      (which == "head" and ("lm_head" in k or "embed" in k))):
+            tensors[k] = tensors[k].float()
+    save_file(tensors, str(folder / "model.safetensors"))
+    cfg, w = plain.read_folder(folder)
+    prompts = random_prompts([5, 17, 40, 70], cfg["vocab_size"], seed=4)
+    want = {f"r{i}": plain.forward(cfg, w, p) for i, p in enumerate(prompts)}
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")                     # "stored in 32-bit": known here
+        runner = runner_for(folder, tiny, torch.bfloat16, 64)
+    for steps in (trace_mixed(prompts, seed=1), trace_tail_decode(prompts, 32)):
+        compare(replay(runner, steps), want, torch.bfloat16, f"{which} in 32-bit")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_captured_decode_steps_follow_the_data(folders, oracle, dtype):
     """Decode-only steps replayed from HIP graphs: every replay is compared with the plain
