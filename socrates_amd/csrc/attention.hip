@@ -460,80 +460,6 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
         }
     }
-    const float c2 = scale * 1.44269504088896340736f;   // scores to base 2
-    const size_t page_stride = (size_t)Hkv * BS * D;
-    const bf16* k_base = k_pool + (size_t)kvh * BS * D;
-    const bf16* v_base = v_pool + (size_t)kvh * BS * D;
-    // Pages of a multiple of 16 keys: a tile lies in one page, so its page is one value for
-    // the whole wave, read on the scalar side, and no lane needs another's.
-    constexpr bool tile_in_page = TP;
-    // Loads must stay in flight until their tile is computed, so nothing touches what they
-    // bring before that: no branch around a load (the two sides would have to be reconciled
-    // in registers behind it), no select on its result. A key that must not be read (outside
-    // what the block's rows can see) is redirected to the first entry of the row's table (a
-    // page of the pool whatever it holds), and its data are replaced by zeros when the tile
-    // is computed, so that what lies in stale slots (inf, NaN) never meets a product.
-    // lookup: the page of the tile (TP: one value for the wave) or of this lane's key (lanes
-    // 0..15 of every lane group hold keys 0..15).
-    auto lookup = [&](int key0) -> int {
-        if constexpr (tile_in_page) {
-            const bool any = key0 < khi && key0 + 16 > kmin;
-            return table[__builtin_amdgcn_readfirstlane(any ? key0 >> bs_shift : 0)];
-        } else {
-            const int key = key0 + li;
-            const bool ok = key >= kmin && key < khi;
-            return table[ok ? key / BS : 0];
-        }
-    };
-    // Global loads of one tile: this lane's K slices and its share of the V tile.
-    auto fetch = [&](int key0, int page, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
-        if constexpr (tile_in_page) {
-            const size_t tile_off = (size_t)page * page_stride + (size_t)((key0 & (BS - 1)) * D);
-            const bf16* krow = k_base + tile_off + li * D;
-#pragma unroll
-            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
-#pragma unroll
-            for (int j = 0; j < V_PER_LANE; ++j) {
-                const int c = (lane + 64 * j) % V_CHUNKS;        // lanes past the tile's chunks reload one of them
-                const int vk = c / (D / 8), part = c % (D / 8);
-                vr[j] = *reinterpret_cast<const uint4*>(v_base + tile_off + vk * D + part * 8);
-            }
-        } else {
-            const int key = key0 + li;
-            const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key % BS) * D;
-#pragma unroll
-            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
-#pragma unroll
-            for (int j = 0; j < V_PER_LANE; ++j) {
-                const int c = (lane + 64 * j) % V_CHUNKS;
-                const int vk = c / (D / 8), part = c % (D / 8);
-                const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
-                vr[j] = *reinterpret_cast<const uint4*>(
-                    v_base + (size_t)vpage * page_stride + (size_t)((key0 + vk) % BS) * D + part * 8);
-            }
-        }
-    };
-
-    // Three tiles are in flight per wave (48 keys). Buffer b holds tiles b, b + 3, b + 6, ...
-    // of the wave's range; the page of a tile is looked up three tiles before its loads are
-    // issued.
-    KFrag kf0, kf1, kf2;
-    uint4 vr0[V_PER_LANE], vr1[V_PER_LANE], vr2[V_PER_LANE];
-    int pa, pb, pc, pg0, pg1, pg2;
-    // Lookups first, then the tile loads: a wait for a lookup then leaves the loads in flight.
-    // Lookups may run past the end of the range (redirected); tile loads do not: the rounds
-    // of the main loop are those in which all three buffers have a tile to load, and what
-    // remains (at most five tiles, two of them still to load) follows without a loop.
-    // FUSED: the first tiles are asked for behind the loads of the row's raw slices and before
-    // the norm and rotation of those, which then run while the tiles are on their way.
-    auto first_tiles = [&] {
-        pa = lookup(klo); pb = lookup(klo + 16); pc = lookup(klo + 32);
-        pg0 = lookup(klo + 48); pg1 = lookup(klo + 64); pg2 = lookup(klo + 80);
-        fetch(klo, pa, kf0, vr0);
-        if (klo + 16 < khi) fetch(klo + 16, pb, kf1, vr1);
-        if (klo + 32 < khi) fetch(klo + 32, pc, kf2, vr2);
-    };
-    if constexpr (!FUSED) first_tiles();
     __shared__ float rope_cs[FUSED ? 4 : 1][FUSED ? D : 1];          // cos [0, D / 2), sin [D / 2, D) of the wave's token
     __shared__ uint4 new_kv[FUSED ? 4 : 1][FUSED ? 2 * (D / 8) : 1]; // the token's key (normed, rotated) and value, by 16-byte part
     if constexpr (FUSED) {
@@ -552,7 +478,6 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
             kraw[kk] = load_qk_slice(row_in + k_at, kk, kb);
         }
         const uint4 vraw = *reinterpret_cast<const uint4*>(row_in + v_at + (lane % (D / 8)) * 8);
-        first_tiles();
         // the token's cosines and sines, from the table (an accurate sincosf in each of a
         // launch's thousands of waves would cost more vector time than the walk itself)
         if (fz.rope_table) {
@@ -648,6 +573,60 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 #pragma unroll
         for (int j = 0; j < DV; ++j) o[rt][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     }
+
+    const float c2 = scale * 1.44269504088896340736f;   // scores to base 2
+    const size_t page_stride = (size_t)Hkv * BS * D;
+    const bf16* k_base = k_pool + (size_t)kvh * BS * D;
+    const bf16* v_base = v_pool + (size_t)kvh * BS * D;
+    // Pages of a multiple of 16 keys: a tile lies in one page, so its page is one value for
+    // the whole wave, read on the scalar side, and no lane needs another's.
+    constexpr bool tile_in_page = TP;
+    // Loads must stay in flight until their tile is computed, so nothing touches what they
+    // bring before that: no branch around a load (the two sides would have to be reconciled
+    // in registers behind it), no select on its result. A key that must not be read (outside
+    // what the block's rows can see) is redirected to the first entry of the row's table (a
+    // page of the pool whatever it holds), and its data are replaced by zeros when the tile
+    // is computed, so that what lies in stale slots (inf, NaN) never meets a product.
+    // lookup: the page of the tile (TP: one value for the wave) or of this lane's key (lanes
+    // 0..15 of every lane group hold keys 0..15).
+    auto lookup = [&](int key0) -> int {
+        if constexpr (tile_in_page) {
+            const bool any = key0 < khi && key0 + 16 > kmin;
+            return table[__builtin_amdgcn_readfirstlane(any ? key0 >> bs_shift : 0)];
+        } else {
+            const int key = key0 + li;
+            const bool ok = key >= kmin && key < khi;
+            return table[ok ? key / BS : 0];
+        }
+    };
+    // Global loads of one tile: this lane's K slices and its share of the V tile.
+    auto fetch = [&](int key0, int page, KFrag& kf, uint4 (&vr)[V_PER_LANE]) {
+        if constexpr (tile_in_page) {
+            const size_t tile_off = (size_t)page * page_stride + (size_t)((key0 & (BS - 1)) * D);
+            const bf16* krow = k_base + tile_off + li * D;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int c = (lane + 64 * j) % V_CHUNKS;        // lanes past the tile's chunks reload one of them
+                const int vk = c / (D / 8), part = c % (D / 8);
+                vr[j] = *reinterpret_cast<const uint4*>(v_base + tile_off + vk * D + part * 8);
+            }
+        } else {
+            const int key = key0 + li;
+            const bf16* krow = k_base + (size_t)page * page_stride + (size_t)(key % BS) * D;
+#pragma unroll
+            for (int kk = 0; kk < QK_STEPS; ++kk) kf.v[kk] = load_qk_slice(krow, kk, kb);
+#pragma unroll
+            for (int j = 0; j < V_PER_LANE; ++j) {
+                const int c = (lane + 64 * j) % V_CHUNKS;
+                const int vk = c / (D / 8), part = c % (D / 8);
+                const int vpage = __shfl(page, vk, SOC_WAVE);                  // from the lane that owns key vk
+                vr[j] = *reinterpret_cast<const uint4*>(
+                    v_base + (size_t)vpage * page_stride + (size_t)((key0 + vk) % BS) * D + part * 8);
+            }
+        }
+    };
 
     // One tile: V to LDS, scores, online softmax, weighted values. MASKED: some key of the
     // tile is hidden from some row of the block (or lies outside the split).
@@ -754,6 +733,20 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
         weighted(pf, alpha, any_rescale);
     };
 
+    // Three tiles are in flight per wave (48 keys). Buffer b holds tiles b, b + 3, b + 6, ...
+    // of the wave's range; the page of a tile is looked up three tiles before its loads are
+    // issued.
+    KFrag kf0, kf1, kf2;
+    uint4 vr0[V_PER_LANE], vr1[V_PER_LANE], vr2[V_PER_LANE];
+    // Lookups first, then the tile loads: a wait for a lookup then leaves the loads in flight.
+    // Lookups may run past the end of the range (redirected); tile loads do not: the rounds
+    // of the main loop are those in which all three buffers have a tile to load, and what
+    // remains (at most five tiles, two of them still to load) follows without a loop.
+    int pa = lookup(klo), pb = lookup(klo + 16), pc = lookup(klo + 32);
+    int pg0 = lookup(klo + 48), pg1 = lookup(klo + 64), pg2 = lookup(klo + 80);
+    fetch(klo, pa, kf0, vr0);
+    if (klo + 16 < khi) fetch(klo + 16, pb, kf1, vr1);
+    if (klo + 32 < khi) fetch(klo + 32, pc, kf2, vr2);
     int key0 = klo;
     for (; key0 + 80 < khi; key0 += 48) {
         tile(key0, kf0, vr0);

@@ -612,6 +612,27 @@ def test_paged_attention_decode_tokens(kernel_sets, dtype, Hq, Hkv, D, bs):
     hip.attention_splits = None
 
 
+@pytest.mark.parametrize("D,bs", [(256, 24), (256, 8), (256, 12), (192, 24), (160, 4), (128, 24)])
+def test_attention_walks_of_large_heads_over_pages_of_any_size(kernel_sets, D, bs):
+    """Head sizes above 128 with pages that hold no multiple of 16 keys (every lane looks its own
+    key's page up), walks long enough for the loop over rounds of three tiles, with one split and
+    with several, a decoded token and a portion; a large scale, so that a key read from the
+    wrong place shows (a reordering of this kernel's first loads once gave wrong sums in just
+    this corner, and nothing in the tests came near it)."""
+    hip, _ = kernel_sets[torch.bfloat16]
+    lens = [1116, 100, 203]
+    slot, dense = make_paged_case(lens, 8, 2, D, bs, torch.bfloat16, seed=D + bs)
+    rows = [0] * 4 + [1] + [2] * 3
+    pos = list(range(1112, 1116)) + [99] + list(range(200, 203))
+    q = rnd((len(rows), 8, D), torch.bfloat16, 5)
+    want = dense_attention(q, dense, rows, pos, 0.3)
+    for splits in (None, (1 << 30, 1), (256, 8), (128, 12)):
+        hip.attention_splits = splits
+        got = hip.paged_attention(q, slot, ctx_for(rows, pos), 0.3)
+        close(got.cpu(), want, torch.bfloat16, atol=3e-2)
+    hip.attention_splits = None
+
+
 @pytest.mark.parametrize("Hq,Hkv,D,bs,norm,rope", [(32, 8, 128, 16, True, True), (16, 1, 64, 32, True, True),
                                                    (8, 2, 32, 8, True, False), (6, 3, 128, 4, False, True),
                                                    (2, 1, 256, 16, True, True), (40, 2, 64, 12, False, False),
